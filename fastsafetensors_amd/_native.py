@@ -1,0 +1,342 @@
+# SPDX-License-Identifier: Apache-2.0
+"""ctypes binding of ``libfstx.so`` (declared in ``include/fstx.h``).
+
+This is the only module that talks to the native library.  It plays the part of
+the reference's pybind11 module ``fastsafetensors.cpp`` (``cpp/ext.cpp:973-1065``,
+typed in ``cpp.pyi``): a reader object with ``submit_read``/``wait_read``, a
+device-buffer handle, and a handful of free functions.  There is no Python or
+CPU substitute for anything in here: if the library is missing, loading raises.
+"""
+
+import ctypes
+import os
+import threading
+from typing import Any, List, Optional, Sequence, Tuple
+
+_LIB_NAME = "libfstx.so"
+_lib: Optional[ctypes.CDLL] = None
+_lib_lock = threading.Lock()
+
+FSTX_ABI_VERSION = 1
+FSTX_BATCH_MAX = 48
+READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
+READ_MODES = {"auto": READ_AUTO, "buffered": READ_BUFFERED, "direct": READ_DIRECT}
+
+
+class NativeError(RuntimeError):
+    """A libfstx call returned a negative status."""
+
+    def __init__(self, what: str, code: int):
+        self.code = code
+        super().__init__(f"{what}: {strerror(code)} (code {code})")
+
+
+class FstxConfig(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("device_id", ctypes.c_int32),
+        ("numa_node", ctypes.c_int32),
+        ("n_threads", ctypes.c_uint32),
+        ("n_streams", ctypes.c_uint32),
+        ("block_bytes", ctypes.c_uint64),
+        ("slots_per_thread", ctypes.c_uint32),
+        ("max_direct_reads", ctypes.c_uint32),
+    ]
+
+
+class FstxMetrics(ctypes.Structure):
+    _fields_ = [
+        (name, ctypes.c_uint64)
+        for name in (
+            "bounce_buffer_bytes",
+            "bytes_read",
+            "bytes_copied",
+            "blocks_buffered",
+            "blocks_direct",
+            "read_ns",
+            "stage_ns",
+            "slot_wait_ns",
+            "direct_fallbacks",
+        )
+    ]
+
+
+class FstxCopyDesc(ctypes.Structure):
+    _fields_ = [("dst", ctypes.c_void_p), ("src", ctypes.c_void_p), ("nbytes", ctypes.c_uint64)]
+
+
+class FstxSliceDesc(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("src", ctypes.c_void_p),
+        ("outer", ctypes.c_uint64),
+        ("seg_bytes", ctypes.c_uint64),
+        ("src_pitch", ctypes.c_uint64),
+    ]
+
+
+# name -> (restype, argtypes); must list every function include/fstx.h declares
+_SIGNATURES = {
+    "fstx_abi_version": (ctypes.c_int, []),
+    "fstx_device_count": (ctypes.c_int, []),
+    "fstx_get_alignment_size": (ctypes.c_int, []),
+    "fstx_get_device_pci_bus": (ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, ctypes.c_int]),
+    "fstx_set_numa_node": (ctypes.c_int, [ctypes.c_int]),
+    "fstx_set_debug_log": (None, [ctypes.c_int]),
+    "fstx_bounce_buffer_bytes": (ctypes.c_uint64, []),
+    "fstx_strerror": (ctypes.c_char_p, [ctypes.c_int64]),
+    "fstx_host_alloc": (ctypes.c_void_p, [ctypes.c_uint64]),
+    "fstx_host_free": (None, [ctypes.c_void_p]),
+    "fstx_ctx_create": (ctypes.c_int, [ctypes.POINTER(FstxConfig), ctypes.POINTER(ctypes.c_void_p)]),
+    "fstx_ctx_destroy": (ctypes.c_int, [ctypes.c_void_p]),
+    "fstx_file_open": (ctypes.c_int64, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int]),
+    "fstx_file_close": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64]),
+    "fstx_submit_read": (
+        ctypes.c_int64,
+        [ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_void_p,
+         ctypes.c_uint64, ctypes.c_uint64],
+    ),
+    "fstx_wait_read": (ctypes.c_int64, [ctypes.c_void_p, ctypes.c_int64]),
+    "fstx_get_metrics": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(FstxMetrics)]),
+    "fstx_realign_copy": (
+        ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]),
+    "fstx_realign_copy_batch": (
+        ctypes.c_int, [ctypes.POINTER(FstxCopyDesc), ctypes.c_uint32, ctypes.c_void_p]),
+    "fstx_slice_copy": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64,
+         ctypes.c_void_p],
+    ),
+    "fstx_slice_copy_batch": (
+        ctypes.c_int, [ctypes.POINTER(FstxSliceDesc), ctypes.c_uint32, ctypes.c_void_p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is None:
+            path = library_path()
+            if not os.path.exists(path):
+                raise ImportError(
+                    f"{path} is missing: build it with `python -m fastsafetensors_amd.build_native` "
+                    "(needs hipcc); this package has no fallback without its HIP library"
+                )
+            handle = ctypes.CDLL(path)
+            for name, (restype, argtypes) in _SIGNATURES.items():
+                fn = getattr(handle, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            got = handle.fstx_abi_version()
+            if got != FSTX_ABI_VERSION:
+                raise ImportError(f"{path}: ABI version {got}, expected {FSTX_ABI_VERSION}")
+            _lib = handle
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return lib().fstx_strerror(int(code)).decode()
+
+
+def _check(what: str, code: int) -> int:
+    if code < 0:
+        raise NativeError(what, code)
+    return code
+
+
+# ---- free functions (names follow the reference's cpp.pyi) ----------------------
+
+
+def device_count() -> int:
+    n = lib().fstx_device_count()
+    return max(n, 0)
+
+
+def is_hip_found() -> bool:
+    return device_count() > 0
+
+
+def get_alignment_size() -> int:
+    return lib().fstx_get_alignment_size()
+
+
+def set_debug_log(enabled: bool) -> None:
+    lib().fstx_set_debug_log(1 if enabled else 0)
+
+
+def get_device_pci_bus(device_id: int) -> str:
+    buf = ctypes.create_string_buffer(64)
+    if lib().fstx_get_device_pci_bus(int(device_id), buf, len(buf)) < 0:
+        return ""
+    return buf.value.decode()
+
+
+def set_numa_node(node: int) -> int:
+    return 0 if lib().fstx_set_numa_node(int(node)) >= 0 else -1
+
+
+def bounce_buffer_bytes() -> int:
+    return int(lib().fstx_bounce_buffer_bytes())
+
+
+def read_buffer(addr: int, length: int) -> bytes:
+    return ctypes.string_at(addr, length)
+
+
+def cpu_malloc(length: int) -> int:
+    return int(lib().fstx_host_alloc(length) or 0)
+
+
+def cpu_free(addr: int) -> None:
+    lib().fstx_host_free(ctypes.c_void_p(addr))
+
+
+class cpp_metrics:
+    """Process-wide counters (``get_cpp_metrics()`` of the reference)."""
+
+    def __init__(self) -> None:
+        self.bounce_buffer_bytes = bounce_buffer_bytes()
+
+
+def get_cpp_metrics() -> cpp_metrics:
+    return cpp_metrics()
+
+
+# ---- device buffer handle ----------------------------------------------------------
+
+
+class DeviceBuffer:
+    """Address range of one file's arena; the ``gds_device_buffer`` of this package.
+
+    ``keepalive`` holds whatever owns the memory (a ``torch.uint8`` tensor), and
+    ``extras`` holds side allocations that must live exactly as long (realigned
+    copies of tensors whose place in the arena is not 16-byte aligned).
+    """
+
+    def __init__(self, base: int, length: int, use_gpu: bool, keepalive: Any = None):
+        self._base = int(base)
+        self._length = int(length)
+        self.use_gpu = bool(use_gpu)
+        self.keepalive = keepalive
+        self.extras: List[Any] = []
+
+    def get_base_address(self) -> int:
+        return self._base
+
+    def get_length(self) -> int:
+        return self._length
+
+    def total_length(self) -> int:
+        return self._length + sum(e.get_length() for e in self.extras)
+
+    def memmove(self, dst_off: int, src_off: int, tmp: "DeviceBuffer", length: int) -> int:
+        """Move ``length`` bytes inside the buffer through ``tmp`` (two kernel copies)."""
+        if max(dst_off, src_off) > self._length or tmp.get_length() < length:
+            return -1
+        if length == 0:
+            return 0
+        try:
+            realign_copy(tmp.get_base_address(), self._base + src_off, length)
+            realign_copy(self._base + dst_off, tmp.get_base_address(), length)
+        except NativeError:
+            return -1
+        return 0
+
+
+# ---- kernels ---------------------------------------------------------------------------
+
+
+def realign_copy(dst: int, src: int, nbytes: int, stream: int = 0) -> None:
+    _check("fstx_realign_copy", lib().fstx_realign_copy(dst, src, nbytes, stream))
+
+
+def realign_copy_batch(jobs: Sequence[Tuple[int, int, int]], stream: int = 0) -> None:
+    """``jobs`` = (dst, src, nbytes) triples; any count (split into launches)."""
+    for i in range(0, len(jobs), FSTX_BATCH_MAX):
+        part = jobs[i : i + FSTX_BATCH_MAX]
+        arr = (FstxCopyDesc * len(part))(*[FstxCopyDesc(d, s, n) for d, s, n in part])
+        _check("fstx_realign_copy_batch", lib().fstx_realign_copy_batch(arr, len(part), stream))
+
+
+def slice_copy(dst: int, src: int, outer: int, seg_bytes: int, src_pitch: int, stream: int = 0) -> None:
+    _check("fstx_slice_copy", lib().fstx_slice_copy(dst, src, outer, seg_bytes, src_pitch, stream))
+
+
+def slice_copy_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:
+    """``jobs`` = (dst, src, outer, seg_bytes, src_pitch) tuples; any count."""
+    for i in range(0, len(jobs), FSTX_BATCH_MAX):
+        part = jobs[i : i + FSTX_BATCH_MAX]
+        arr = (FstxSliceDesc * len(part))(*[FstxSliceDesc(*j) for j in part])
+        _check("fstx_slice_copy_batch", lib().fstx_slice_copy_batch(arr, len(part), stream))
+
+
+# ---- reader ------------------------------------------------------------------------------
+
+
+class Reader:
+    """One copy pipeline: worker threads, pinned ring and copy streams."""
+
+    def __init__(
+        self,
+        device_id: int,
+        numa_node: int = -1,
+        n_threads: int = 0,
+        n_streams: int = 0,
+        block_bytes: int = 0,
+        slots_per_thread: int = 0,
+        max_direct_reads: int = 0,
+    ):
+        cfg = FstxConfig(
+            ctypes.sizeof(FstxConfig), device_id, numa_node, n_threads, n_streams, block_bytes,
+            slots_per_thread, max_direct_reads,
+        )
+        handle = ctypes.c_void_p()
+        _check("fstx_ctx_create", lib().fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(handle)))
+        self._ctx: Optional[ctypes.c_void_p] = handle
+
+    def _h(self) -> ctypes.c_void_p:
+        if self._ctx is None:
+            raise RuntimeError("reader is closed")
+        return self._ctx
+
+    def open(self, path: str, mode: int = READ_AUTO) -> int:
+        return _check(f"fstx_file_open({path})", lib().fstx_file_open(self._h(), os.fsencode(path), mode))
+
+    def close_file(self, file: int) -> None:
+        _check("fstx_file_close", lib().fstx_file_close(self._h(), file))
+
+    def submit_read(self, file: int, dst: DeviceBuffer, offset: int, length: int, ptr_off: int) -> int:
+        return _check(
+            "fstx_submit_read",
+            lib().fstx_submit_read(
+                self._h(), file, offset, length, dst.get_base_address(), dst.get_length(), ptr_off
+            ),
+        )
+
+    def wait_read(self, request: int) -> int:
+        return _check("fstx_wait_read", lib().fstx_wait_read(self._h(), request))
+
+    def metrics(self) -> FstxMetrics:
+        m = FstxMetrics()
+        _check("fstx_get_metrics", lib().fstx_get_metrics(self._h(), ctypes.byref(m)))
+        return m
+
+    def close(self) -> None:
+        if self._ctx is not None:
+            ctx, self._ctx = self._ctx, None
+            lib().fstx_ctx_destroy(ctx)
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,251 @@
+# SPDX-License-Identifier: Apache-2.0
+"""The ``"mi355x"`` copier: safetensors file -> one HBM arena per file.
+
+It sits where the reference's ``NoGdsFileCopier`` sits (``copier/nogds.py:15-118``)
+and keeps that copier's contract, but hands the work to ``libfstx``:
+
+* ``submit_io`` allocates the arena and enqueues the file's data section on the
+  shared read pipeline (O_DIRECT or page-cache reads into a pinned ring,
+  asynchronous copies on several HIP streams);
+* ``wait_io`` drains the requests, realigns what needs realigning with the
+  realign-copy kernel, and returns zero-copy tensor views.
+
+Arena layouts
+-------------
+``direct`` (default)
+    Arena byte ``lead + i`` holds data-section byte ``i``.  The DMA engine
+    places bytes at any address for free, so a header whose length is not a
+    multiple of 16 costs nothing.  ``lead`` (0..15) is chosen so that as many
+    tensor bytes as possible start on a 16-byte boundary; the few tensors that
+    still do not are copied to an aligned side buffer by one batched kernel
+    launch.
+``window``
+    The arena holds the 4 KiB-aligned file window that contains the data
+    section, header tail included, exactly as an O_DIRECT or GDS read delivers
+    it (reference: ``copier/gds.py:61-78``).  When ``header_length % 16 != 0``
+    every tensor is then misaligned and the whole section is shifted into a
+    fresh aligned arena by the realign-copy kernel -- the job the reference does
+    with ``gds_device_buffer.memmove`` through a 1 GiB temporary
+    (``copier/gds.py:138-159``).
+"""
+
+import os
+from typing import Dict, List, Optional, Tuple
+
+from .. import _native
+from ..common import SafeTensorsMetadata, TensorFrame
+from ..frameworks import FrameworkOpBase, TensorBase
+from ..st_types import Device, DeviceType, DType, dtype_storage_align
+from .base import CopierInterface
+from .registry import CopierConstructFunc, register_copier_constructor
+
+PTR_ALIGN = 16
+WINDOW_ALIGN = 4096
+LAYOUTS = ("direct", "window")
+
+
+def _align_up(v: int, a: int) -> int:
+    return -(-v // a) * a
+
+
+def pick_lead(frames: List[TensorFrame], align: int = PTR_ALIGN) -> int:
+    """Offset 0..align-1 of the data section inside the arena that puts the most
+    tensor bytes on an ``align`` boundary (ties go to the smallest offset)."""
+    weight = [0] * align
+    for f in frames:
+        weight[-f.data_offsets[0] % align] += f.nbytes
+    return max(range(align), key=lambda lead: (weight[lead], -lead))
+
+
+class MI355XFileCopier(CopierInterface):
+    def __init__(
+        self,
+        metadata: SafeTensorsMetadata,
+        device: Device,
+        reader: _native.Reader,
+        framework: FrameworkOpBase,
+        read_mode: str = "auto",
+        layout: str = "direct",
+    ):
+        if device.type == DeviceType.CPU:
+            raise Exception("MI355XFileCopier: needs a HIP device; device='cpu' is not served")
+        if layout not in LAYOUTS:
+            raise ValueError(f"MI355XFileCopier: unknown layout {layout!r}, expected one of {LAYOUTS}")
+        if read_mode not in _native.READ_MODES:
+            raise ValueError(f"MI355XFileCopier: unknown read_mode {read_mode!r}")
+        self.metadata = metadata
+        self.device = device
+        self.reader = reader
+        self.framework = framework
+        self.layout = layout
+        self.file: Optional[int] = reader.open(metadata.src, _native.READ_MODES[read_mode])
+        self.reqs: List[int] = []
+        self.data_at = 0  # arena offset of data-section byte 0
+
+    # -- submit -------------------------------------------------------------------
+    def submit_io(self, use_buf_register: bool, max_copy_block_size: int) -> _native.DeviceBuffer:
+        meta = self.metadata
+        if self.layout == "window":
+            first = meta.header_length - meta.header_length % WINDOW_ALIGN
+            self.data_at = meta.header_length - first
+        else:
+            first = meta.header_length
+            self.data_at = pick_lead(list(meta.tensors.values()))
+        total = meta.size_bytes - first
+        lead = self.data_at if self.layout == "direct" else 0
+        gbuf = self.framework.alloc_tensor_memory(lead + total, self.device)
+        try:
+            done = 0
+            while done < total:
+                length = min(total - done, max_copy_block_size)
+                self.reqs.append(
+                    self.reader.submit_read(self.file, gbuf, first + done, length, lead + done)
+                )
+                done += length
+        except Exception:
+            self._drain()
+            self.framework.free_tensor_memory(gbuf, self.device)
+            raise
+        return gbuf
+
+    def _drain(self) -> List[Tuple[int, Exception]]:
+        failed = []
+        for req in self.reqs:
+            try:
+                self.reader.wait_read(req)
+            except _native.NativeError as e:
+                failed.append((req, e))
+        self.reqs = []
+        if self.file is not None:
+            self.reader.close_file(self.file)
+            self.file = None
+        return failed
+
+    # -- wait -----------------------------------------------------------------------
+    def wait_io(
+        self, gbuf: _native.DeviceBuffer, dtype: DType = DType.AUTO, noalign: bool = False
+    ) -> Dict[str, TensorBase]:
+        failed = self._drain()
+        if failed:
+            raise Exception(
+                f"wait_io: read failed, file={self.metadata.src}, "
+                + ", ".join(f"req {r}: {e}" for r, e in failed)
+            )
+        if dtype != DType.AUTO:
+            raise NotImplementedError(
+                "dtype conversion on load is outside this loader's scope; pass DType.AUTO"
+            )
+        meta, fw = self.metadata, self.framework
+        arena, data_at = gbuf, self.data_at
+        if self.layout == "window" and not noalign and data_at % PTR_ALIGN and meta.data_length:
+            # shift the whole data section onto a 16-byte boundary, out of place
+            lead = pick_lead(list(meta.tensors.values()))
+            fresh = fw.alloc_side_memory(gbuf, lead + meta.data_length, self.device)
+            _native.realign_copy(
+                fresh.get_base_address() + lead,
+                gbuf.get_base_address() + data_at,
+                meta.data_length,
+                self._stream(),
+            )
+            fw.synchronize(self.device)
+            fw.shrink_tensor_memory(gbuf)
+            arena, data_at = fresh, lead
+
+        # tensors that still start off-boundary move to an aligned side buffer
+        base = arena.get_base_address()
+        need = {}
+        for name, frame in meta.tensors.items():
+            want = dtype_storage_align(frame.dtype) if noalign else PTR_ALIGN
+            if frame.nbytes and (base + data_at + frame.data_offsets[0]) % want:
+                need[name] = frame
+        side = None
+        placed: Dict[str, int] = {}
+        if need:
+            cursor = 0
+            for name, frame in need.items():
+                placed[name] = cursor
+                cursor += _align_up(frame.nbytes, PTR_ALIGN)
+            side = fw.alloc_side_memory(gbuf, cursor, self.device)
+            _native.realign_copy_batch(
+                [
+                    (side.get_base_address() + placed[n], base + data_at + f.data_offsets[0], f.nbytes)
+                    for n, f in need.items()
+                ],
+                self._stream(),
+            )
+            fw.synchronize(self.device)
+
+        tensors: Dict[str, TensorBase] = {}
+        for name, frame in meta.tensors.items():
+            if name in placed:
+                tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
+            else:
+                tensors[name] = fw.view_tensor(arena, data_at + frame.data_offsets[0], frame, self.device)
+        return tensors
+
+    def _stream(self) -> int:
+        import torch
+
+        return torch.cuda.current_stream().cuda_stream
+
+    def __del__(self) -> None:
+        try:
+            if self.reqs or self.file is not None:
+                self._drain()
+        except Exception:
+            pass
+
+
+def _default_numa_node(device: Device) -> int:
+    from ..common import get_device_numa_node
+
+    node = get_device_numa_node(device.index if device.index is not None else 0)
+    return -1 if node is None or node < 0 else node
+
+
+@register_copier_constructor("mi355x")
+def new_mi355x_file_copier(
+    device: Device,
+    bbuf_size_kb: int = 16 * 1024,
+    max_threads: int = 16,
+    framework: Optional[FrameworkOpBase] = None,
+    read_mode: Optional[str] = None,
+    layout: Optional[str] = None,
+    block_size_kb: Optional[int] = None,
+    n_streams: int = 0,
+    slots_per_thread: int = 0,
+    max_direct_reads: int = 0,
+    numa_node: Optional[int] = None,
+    **kwargs,
+) -> CopierConstructFunc:
+    """One read pipeline (threads, pinned ring, streams) shared by every file of a
+    loader, as the reference shares one ``nogds_file_reader`` (``copier/nogds.py:107-116``).
+
+    ``bbuf_size_kb`` is accepted for signature compatibility; the ring is sized
+    ``max_threads * slots_per_thread * block_size_kb`` instead, because 1 MiB
+    slots (the reference's default split) cap the host-to-device link well
+    below its peak.
+    """
+    if device.type == DeviceType.CPU:
+        raise Exception("copier 'mi355x' needs a HIP device; device='cpu' is not served")
+    if _native.device_count() <= 0:
+        raise Exception("[FAIL] no HIP device is visible to libfstx")
+    read_mode = read_mode or os.environ.get("FSTX_READ_MODE", "auto")
+    layout = layout or os.environ.get("FSTX_LAYOUT", "direct")
+    block_kb = block_size_kb or int(os.environ.get("FSTX_BLOCK_KB", "4096"))
+    reader = _native.Reader(
+        device.index if device.index is not None else 0,
+        numa_node=_default_numa_node(device) if numa_node is None else numa_node,
+        n_threads=max_threads,
+        n_streams=n_streams,
+        block_bytes=block_kb * 1024,
+        slots_per_thread=slots_per_thread,
+        max_direct_reads=max_direct_reads,
+    )
+
+    def construct(metadata: SafeTensorsMetadata, device: Device, framework: FrameworkOpBase) -> CopierInterface:
+        return MI355XFileCopier(metadata, device, reader, framework, read_mode=read_mode, layout=layout)
+
+    construct.reader = reader  # type: ignore[attr-defined]
+    construct.close = reader.close  # type: ignore[attr-defined]
+    return construct

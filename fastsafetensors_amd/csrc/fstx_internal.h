@@ -1,0 +1,47 @@
+// SPDX-License-Identifier: Apache-2.0
+//
+// Seams inside libfstx: the pipeline (fstx_pipeline.cpp) is plain C++ and
+// reaches the GPU runtime only through the few calls declared in fstx_dev.
+// The shipped library binds them to HIP (fstx_device_hip.cpp).  The host-side
+// unit tests link the same pipeline source against an in-memory stand-in so
+// that thread sanitizers can run without a GPU; that stand-in is not part of
+// the shipped library.
+#ifndef FSTX_INTERNAL_H
+#define FSTX_INTERNAL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fstx_dev {
+
+typedef void *stream_t;
+typedef void *event_t;
+
+// every call returns 0 or a negative fstx status
+int device_count();
+int set_device(int device_id);
+int pci_bus_id(int device_id, char *out, int len);
+int host_alloc(void **out, size_t bytes);   // pinned, device-visible host memory
+int host_free(void *p);
+int stream_create(stream_t *out);
+int stream_destroy(stream_t s);
+int stream_sync(stream_t s);
+int event_create(event_t *out);
+int event_destroy(event_t e);
+int event_record(event_t e, stream_t s);
+int event_ready(event_t e);                 // 1 done, 0 still running, <0 error
+int event_sync(event_t e);
+int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stream_t s);
+
+} // namespace fstx_dev
+
+namespace fstx_internal {
+
+int check_launch(const char *what);  // hipGetLastError -> 0 / -FSTX_E_HIP
+bool debug_enabled();
+void debug(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void note_bounce_bytes(int64_t delta); // process-wide pinned ring accounting
+
+} // namespace fstx_internal
+
+#endif

@@ -1,0 +1,685 @@
+// SPDX-License-Identifier: Apache-2.0
+//
+// File -> pinned ring -> HBM copy pipeline.
+//
+// What it replaces: nogds_file_reader of the reference (cpp/ext.cpp:648-806,
+// cpp/ext.hpp:155-185), which starts one thread per request and, inside it,
+// alternates a page-cache pread with a synchronous host-to-device memcpy.
+//
+// Shape of this one:
+//   * a fixed pool of worker threads, pinned to the GPU's NUMA node;
+//   * every request is cut into blocks of `block_bytes` on 4 KiB file
+//     boundaries; workers pull blocks from one FIFO, so a single large file
+//     is read by all workers at once;
+//   * each worker cycles through its own slots of a pinned ring that is
+//     allocated once per context; after the read it enqueues an asynchronous
+//     host-to-device copy and an event on one of the shared copy streams and
+//     moves on to its next slot, so the copy of block k overlaps the read of
+//     block k+1 (the event is waited only when the slot comes round again);
+//   * a block is read either from the page cache straight into the ring, or
+//     with O_DIRECT into an ordinary aligned staging block and then moved
+//     into the ring.  O_DIRECT cannot target the ring itself: device-visible
+//     pinned memory is not backed by pages the block layer can pin, and
+//     the read fails with EFAULT.  In AUTO mode the choice is made per block
+//     from mincore() residency.
+//
+// Nothing here touches the GPU runtime directly; see fstx_internal.h.
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include <errno.h>
+#include <fcntl.h>
+#include <sched.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include "fstx.h"
+#include "fstx_internal.h"
+
+namespace {
+
+constexpr uint64_t kPage = 4096;
+constexpr uint64_t kDefaultBlock = 4ull << 20;
+constexpr double kResidentEnough = 0.95;
+
+inline uint64_t align_down(uint64_t v, uint64_t a) { return v - v % a; }
+inline uint64_t align_up(uint64_t v, uint64_t a) { return align_down(v + a - 1, a); }
+inline uint64_t now_ns() {
+    return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+               std::chrono::steady_clock::now().time_since_epoch())
+        .count();
+}
+
+std::atomic<int> g_debug{0};
+std::atomic<int64_t> g_bounce_bytes{0};
+
+// ---- NUMA ------------------------------------------------------------------
+
+// CPUs of a node from sysfs ("0-15,32-47"); empty when unknown
+std::vector<int> node_cpus(int node) {
+    std::vector<int> cpus;
+    char path[96];
+    std::snprintf(path, sizeof path, "/sys/devices/system/node/node%d/cpulist", node);
+    FILE *f = std::fopen(path, "r");
+    if (!f) return cpus;
+    char buf[4096];
+    if (std::fgets(buf, sizeof buf, f)) {
+        char *p = buf;
+        while (*p && *p != '\n') {
+            char *end;
+            long a = std::strtol(p, &end, 10);
+            if (end == p) break;
+            long b = a;
+            p = end;
+            if (*p == '-') {
+                b = std::strtol(p + 1, &end, 10);
+                p = end;
+            }
+            for (long c = a; c <= b && c < CPU_SETSIZE; ++c) cpus.push_back((int)c);
+            if (*p == ',') ++p;
+        }
+    }
+    std::fclose(f);
+    return cpus;
+}
+
+int bind_thread_to_node(int node) {
+    if (node < 0) return 0;
+    std::vector<int> cpus = node_cpus(node);
+    if (cpus.empty()) return -ENODEV;
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    for (int c : cpus) CPU_SET(c, &set);
+    if (sched_setaffinity(0, sizeof set, &set) != 0) return -errno;
+#ifdef SYS_set_mempolicy
+    if (node < 64) {
+        // MPOL_PREFERRED = 1: allocate on this node while it has room
+        unsigned long mask = 1ul << node;
+        (void)syscall(SYS_set_mempolicy, 1, &mask, sizeof(mask) * 8);
+    }
+#endif
+    return 0;
+}
+
+// ---- data model ------------------------------------------------------------
+
+struct FileEntry {
+    int fd_buffered = -1;
+    int fd_direct = -1; // -1: the filesystem refused O_DIRECT
+    int mode = FSTX_READ_AUTO;
+    uint64_t size = 0;
+    void *map = nullptr; // read-only mapping, used only for mincore()
+    std::atomic<bool> direct_ok{true};
+    std::atomic<int64_t> open_requests{0};
+};
+
+struct Request {
+    int64_t id = 0;
+    std::shared_ptr<FileEntry> file;
+    uint64_t length = 0;
+    std::atomic<uint64_t> blocks_left{0};
+    std::atomic<int64_t> error{0};      // first negative status seen by a worker
+    std::atomic<uint64_t> stream_mask{0}; // copy streams that carry blocks of this request
+};
+
+struct Block {
+    std::shared_ptr<Request> req;
+    uint64_t file_off; // first payload byte in the file
+    uint64_t len;      // payload bytes
+    char *dev;         // device address of the first payload byte
+};
+
+struct Slot {
+    char *host = nullptr;
+    fstx_dev::event_t ev = nullptr;
+    bool pending = false; // an async copy out of this slot may still be running
+};
+
+// counting semaphore bounding concurrent O_DIRECT preads
+class Gate {
+  public:
+    explicit Gate(uint32_t n) : free_(n) {}
+    void enter() {
+        std::unique_lock<std::mutex> lk(m_);
+        cv_.wait(lk, [&] { return free_ > 0; });
+        --free_;
+    }
+    void leave() {
+        {
+            std::lock_guard<std::mutex> lk(m_);
+            ++free_;
+        }
+        cv_.notify_one();
+    }
+
+  private:
+    std::mutex m_;
+    std::condition_variable cv_;
+    uint32_t free_;
+};
+
+struct Counters {
+    std::atomic<uint64_t> bytes_read{0}, bytes_copied{0}, blocks_buffered{0}, blocks_direct{0},
+        read_ns{0}, stage_ns{0}, slot_wait_ns{0}, direct_fallbacks{0};
+};
+
+} // namespace
+
+struct fstx_ctx {
+    fstx_config cfg{};
+    uint64_t ring_bytes = 0;
+    char *ring = nullptr;
+    std::vector<fstx_dev::stream_t> streams;
+    std::vector<std::vector<Slot>> slots; // [thread][slot]
+    std::vector<std::thread> workers;
+    std::unique_ptr<Gate> direct_gate;
+
+    std::mutex q_mutex;
+    std::condition_variable q_cv;
+    std::deque<Block> queue;
+    bool closing = false;
+
+    std::mutex done_mutex;
+    std::condition_variable done_cv;
+
+    std::mutex table_mutex;
+    std::map<int64_t, std::shared_ptr<FileEntry>> files;
+    std::map<int64_t, std::shared_ptr<Request>> requests;
+    int64_t next_file = 1;
+    int64_t next_request = 1;
+
+    Counters ctr;
+    std::atomic<int64_t> fault_after{-1}; // test hook: fail the n-th block read with EIO
+};
+
+namespace {
+
+// ---- reading one block -------------------------------------------------------
+
+// pread until `want` bytes arrived, EOF or error; returns bytes or -errno
+int64_t pread_full(int fd, char *buf, uint64_t want, uint64_t off) {
+    uint64_t got = 0;
+    while (got < want) {
+        ssize_t c = pread(fd, buf + got, want - got, (off_t)(off + got));
+        if (c < 0) {
+            if (errno == EINTR) continue;
+            return -(int64_t)errno;
+        }
+        if (c == 0) break;
+        got += (uint64_t)c;
+    }
+    return (int64_t)got;
+}
+
+bool block_is_cached(const FileEntry &f, uint64_t lo, uint64_t hi) {
+    if (!f.map) return false;
+    lo = align_down(lo, kPage);
+    hi = std::min(align_up(hi, kPage), align_up(f.size, kPage));
+    if (hi <= lo) return true;
+    const size_t pages = (size_t)((hi - lo) / kPage);
+    unsigned char stack_vec[2048];
+    std::vector<unsigned char> heap_vec;
+    unsigned char *vec = stack_vec;
+    if (pages > sizeof stack_vec) {
+        heap_vec.resize(pages);
+        vec = heap_vec.data();
+    }
+    if (mincore(static_cast<char *>(f.map) + lo, hi - lo, vec) != 0) return false;
+    size_t in = 0;
+    for (size_t i = 0; i < pages; ++i) in += vec[i] & 1;
+    return (double)in >= kResidentEnough * (double)pages;
+}
+
+struct Worker {
+    fstx_ctx *ctx;
+    uint32_t index;
+    char *stage = nullptr; // ordinary page-backed memory for O_DIRECT reads
+
+    ~Worker() { std::free(stage); }
+
+    // Fill `slot` so that payload byte i sits at slot + (file_off - window) + i.
+    // Returns the in-slot offset of the payload or a negative status.
+    int64_t fill(const Block &b, Slot &slot) {
+        FileEntry &f = *b.req->file;
+        const uint64_t window = align_down(b.file_off, kPage);
+        const uint64_t in_slot = b.file_off - window;
+
+        int64_t hook = ctx->fault_after.load(std::memory_order_relaxed);
+        if (hook >= 0 && ctx->fault_after.fetch_sub(1) == 0) return -EIO;
+
+        bool direct = false;
+        if (f.fd_direct >= 0 && f.direct_ok.load(std::memory_order_relaxed)) {
+            if (f.mode == FSTX_READ_DIRECT) direct = true;
+            else if (f.mode == FSTX_READ_AUTO)
+                direct = !block_is_cached(f, b.file_off, b.file_off + b.len);
+        } else if (f.mode == FSTX_READ_DIRECT) {
+            ctx->ctr.direct_fallbacks.fetch_add(1, std::memory_order_relaxed);
+        }
+
+        if (direct) {
+            if (!stage && posix_memalign(reinterpret_cast<void **>(&stage), kPage,
+                                         ctx->cfg.block_bytes + kPage) != 0) {
+                stage = nullptr;
+                return -ENOMEM;
+            }
+            const uint64_t want = align_up(in_slot + b.len, kPage);
+            ctx->direct_gate->enter();
+            uint64_t t0 = now_ns();
+            int64_t got = pread_full(f.fd_direct, stage, want, window);
+            uint64_t t1 = now_ns();
+            ctx->direct_gate->leave();
+            if (got == -EINVAL || got == -EFAULT || got == -EOPNOTSUPP) {
+                // this file cannot do O_DIRECT after all; stay buffered from here on
+                f.direct_ok.store(false, std::memory_order_relaxed);
+                ctx->ctr.direct_fallbacks.fetch_add(1, std::memory_order_relaxed);
+                direct = false;
+            } else {
+                if (got < 0) return got;
+                if ((uint64_t)got < in_slot + b.len) return -FSTX_E_SHORT_READ;
+                std::memcpy(slot.host + in_slot, stage + in_slot, b.len);
+                uint64_t t2 = now_ns();
+                ctx->ctr.read_ns.fetch_add(t1 - t0, std::memory_order_relaxed);
+                ctx->ctr.stage_ns.fetch_add(t2 - t1, std::memory_order_relaxed);
+                ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
+            }
+        }
+        if (!direct) {
+            uint64_t t0 = now_ns();
+            int64_t got = pread_full(f.fd_buffered, slot.host + in_slot, b.len, b.file_off);
+            ctx->ctr.read_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
+            if (got < 0) return got;
+            if ((uint64_t)got < b.len) return -FSTX_E_SHORT_READ;
+            ctx->ctr.blocks_buffered.fetch_add(1, std::memory_order_relaxed);
+        }
+        ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
+        return (int64_t)in_slot;
+    }
+
+    void run() {
+        bind_thread_to_node(ctx->cfg.numa_node);
+        int dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
+        std::vector<Slot> &mine = ctx->slots[index];
+        const uint32_t stream_ix = index % (uint32_t)ctx->streams.size();
+        fstx_dev::stream_t stream = ctx->streams[stream_ix];
+        size_t turn = 0;
+        for (;;) {
+            Block b;
+            {
+                std::unique_lock<std::mutex> lk(ctx->q_mutex);
+                ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty(); });
+                if (ctx->queue.empty()) break; // closing and drained
+                b = std::move(ctx->queue.front());
+                ctx->queue.pop_front();
+            }
+            int64_t status = dev_rc;
+            // once a request has failed, its remaining blocks are only counted off
+            if (status == 0 && b.req->error.load(std::memory_order_relaxed) == 0) {
+                Slot &slot = mine[turn];
+                turn = (turn + 1) % mine.size();
+                if (slot.pending) {
+                    if (fstx_dev::event_ready(slot.ev) != 1) {
+                        uint64_t t0 = now_ns();
+                        status = fstx_dev::event_sync(slot.ev);
+                        ctx->ctr.slot_wait_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
+                    }
+                    slot.pending = false;
+                }
+                if (status == 0) {
+                    int64_t in_slot = fill(b, slot);
+                    if (in_slot < 0) status = in_slot;
+                    else {
+                        status = fstx_dev::copy_to_device_async(b.dev, slot.host + in_slot, b.len, stream);
+                        if (status == 0) {
+                            slot.pending = true;
+                            status = fstx_dev::event_record(slot.ev, stream);
+                            b.req->stream_mask.fetch_or(1ull << stream_ix, std::memory_order_relaxed);
+                            ctx->ctr.bytes_copied.fetch_add(b.len, std::memory_order_relaxed);
+                        }
+                    }
+                }
+            }
+            if (status < 0) {
+                int64_t none = 0;
+                b.req->error.compare_exchange_strong(none, status);
+            }
+            if (b.req->blocks_left.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+                std::lock_guard<std::mutex> lk(ctx->done_mutex);
+                ctx->done_cv.notify_all();
+            }
+        }
+        // leave no copy in flight that still reads this worker's slots
+        for (Slot &s : mine)
+            if (s.pending) {
+                fstx_dev::event_sync(s.ev);
+                s.pending = false;
+            }
+    }
+};
+
+void release_file(FileEntry &f) {
+    if (f.map) munmap(f.map, f.size);
+    if (f.fd_direct >= 0) close(f.fd_direct);
+    if (f.fd_buffered >= 0) close(f.fd_buffered);
+    f.map = nullptr;
+    f.fd_direct = f.fd_buffered = -1;
+}
+
+} // namespace
+
+// ---- library-wide helpers ----------------------------------------------------
+
+namespace fstx_internal {
+bool debug_enabled() { return g_debug.load(std::memory_order_relaxed) != 0; }
+void debug(const char *fmt, ...) {
+    if (!debug_enabled()) return;
+    va_list ap;
+    va_start(ap, fmt);
+    std::fputs("[fstx] ", stderr);
+    std::vfprintf(stderr, fmt, ap);
+    std::fputc('\n', stderr);
+    va_end(ap);
+}
+void note_bounce_bytes(int64_t delta) { g_bounce_bytes.fetch_add(delta); }
+} // namespace fstx_internal
+
+extern "C" {
+
+int fstx_abi_version(void) { return FSTX_ABI_VERSION; }
+int fstx_device_count(void) { return fstx_dev::device_count(); }
+int fstx_get_alignment_size(void) { return (int)kPage; }
+void fstx_set_debug_log(int enabled) { g_debug.store(enabled ? 1 : 0); }
+uint64_t fstx_bounce_buffer_bytes(void) { return (uint64_t)g_bounce_bytes.load(); }
+
+int fstx_get_device_pci_bus(int device_id, char *out, int len) {
+    if (!out || len < 13) return -FSTX_E_INVAL;
+    out[0] = 0;
+    return fstx_dev::pci_bus_id(device_id, out, len);
+}
+
+int fstx_set_numa_node(int numa_node) {
+    int rc = bind_thread_to_node(numa_node);
+    return rc < 0 ? rc : 0;
+}
+
+void *fstx_host_alloc(uint64_t length) {
+    void *p = nullptr;
+    if (posix_memalign(&p, kPage, length ? length : 1) != 0) return nullptr;
+    return p;
+}
+void fstx_host_free(void *p) { std::free(p); }
+
+const char *fstx_strerror(int64_t code) {
+    if (code >= 0) return "ok";
+    int64_t c = -code;
+    switch (c) {
+    case FSTX_E_INVAL: return "fstx: invalid argument";
+    case FSTX_E_HIP: return "fstx: HIP runtime call failed";
+    case FSTX_E_RANGE: return "fstx: range exceeds the device buffer";
+    case FSTX_E_SHORT_READ: return "fstx: file ended before the requested range";
+    case FSTX_E_NO_REQ: return "fstx: unknown request or file handle";
+    case FSTX_E_CLOSED: return "fstx: context is shutting down";
+    case FSTX_E_NO_DEVICE: return "fstx: no HIP device visible";
+    case FSTX_E_TOO_MANY: return "fstx: batch exceeds FSTX_BATCH_MAX";
+    default: break;
+    }
+    if (c < FSTX_E_BASE) return std::strerror((int)c);
+    return "fstx: unknown error";
+}
+
+// ---- context -----------------------------------------------------------------
+
+int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
+    if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
+    *out = nullptr;
+    fstx_config cfg = *cfg_in;
+    if (cfg.n_threads == 0) cfg.n_threads = 8;
+    if (cfg.n_streams == 0) cfg.n_streams = 4;
+    if (cfg.block_bytes == 0) cfg.block_bytes = kDefaultBlock;
+    if (cfg.slots_per_thread == 0) cfg.slots_per_thread = 2;
+    if (cfg.max_direct_reads == 0) cfg.max_direct_reads = 4;
+    if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 ||
+        cfg.slots_per_thread > 64)
+        return -FSTX_E_INVAL;
+    cfg.n_streams = std::min(cfg.n_streams, cfg.n_threads);
+
+    int n_dev = fstx_dev::device_count();
+    if (n_dev < 0) return n_dev;
+    if (cfg.device_id < 0 || cfg.device_id >= n_dev) return -FSTX_E_INVAL;
+    int rc = fstx_dev::set_device(cfg.device_id);
+    if (rc < 0) return rc;
+
+    std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
+    ctx->cfg = cfg;
+    ctx->direct_gate.reset(new Gate(cfg.max_direct_reads));
+    if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
+
+    // each slot holds one block plus the 4 KiB lead-in of an unaligned start
+    const uint64_t slot_bytes = cfg.block_bytes + kPage;
+    const uint64_t n_slots = (uint64_t)cfg.n_threads * cfg.slots_per_thread;
+    ctx->ring_bytes = slot_bytes * n_slots;
+    {
+        // allocate (and thereby place) the ring while this thread prefers the node
+        cpu_set_t saved;
+        bool restore = cfg.numa_node >= 0 && sched_getaffinity(0, sizeof saved, &saved) == 0;
+        if (cfg.numa_node >= 0) bind_thread_to_node(cfg.numa_node);
+        void *p = nullptr;
+        rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
+        if (restore) {
+            sched_setaffinity(0, sizeof saved, &saved);
+#ifdef SYS_set_mempolicy
+            (void)syscall(SYS_set_mempolicy, 0, nullptr, 0); // MPOL_DEFAULT
+#endif
+        }
+        if (rc < 0) return rc;
+        ctx->ring = static_cast<char *>(p);
+        fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
+    }
+    auto fail = [&](int code) {
+        for (auto &per : ctx->slots)
+            for (Slot &s : per)
+                if (s.ev) fstx_dev::event_destroy(s.ev);
+        for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
+        fstx_dev::host_free(ctx->ring);
+        fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
+        return code;
+    };
+    for (uint32_t i = 0; i < cfg.n_streams; ++i) {
+        fstx_dev::stream_t s = nullptr;
+        if ((rc = fstx_dev::stream_create(&s)) < 0) return fail(rc);
+        ctx->streams.push_back(s);
+    }
+    ctx->slots.resize(cfg.n_threads);
+    for (uint32_t t = 0; t < cfg.n_threads; ++t) {
+        for (uint32_t k = 0; k < cfg.slots_per_thread; ++k) {
+            Slot s;
+            s.host = ctx->ring + ((uint64_t)t * cfg.slots_per_thread + k) * slot_bytes;
+            if ((rc = fstx_dev::event_create(&s.ev)) < 0) return fail(rc);
+            ctx->slots[t].push_back(s);
+        }
+    }
+    fstx_ctx *raw = ctx.release();
+    for (uint32_t t = 0; t < cfg.n_threads; ++t) {
+        raw->workers.emplace_back([raw, t] {
+            Worker w{raw, t};
+            w.run();
+        });
+    }
+    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu", cfg.device_id,
+                         cfg.n_threads, cfg.n_streams, (unsigned long long)cfg.block_bytes,
+                         (unsigned long long)raw->ring_bytes);
+    *out = raw;
+    return 0;
+}
+
+int fstx_ctx_destroy(fstx_ctx *ctx) {
+    if (!ctx) return -FSTX_E_INVAL;
+    {
+        std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        ctx->closing = true;
+    }
+    ctx->q_cv.notify_all();
+    for (std::thread &t : ctx->workers) t.join(); // workers drain the queue first
+    fstx_dev::set_device(ctx->cfg.device_id);
+    for (auto s : ctx->streams) fstx_dev::stream_sync(s);
+    for (auto &per : ctx->slots)
+        for (Slot &s : per) fstx_dev::event_destroy(s.ev);
+    for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
+    for (auto &kv : ctx->files) release_file(*kv.second);
+    fstx_dev::host_free(ctx->ring);
+    fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
+    delete ctx;
+    return 0;
+}
+
+// ---- files ---------------------------------------------------------------------
+
+int64_t fstx_file_open(fstx_ctx *ctx, const char *path, int mode) {
+    if (!ctx || !path || mode < FSTX_READ_AUTO || mode > FSTX_READ_DIRECT) return -FSTX_E_INVAL;
+    auto f = std::make_shared<FileEntry>();
+    f->mode = mode;
+    f->fd_buffered = open(path, O_RDONLY | O_CLOEXEC);
+    if (f->fd_buffered < 0) return -(int64_t)errno;
+    struct stat st;
+    if (fstat(f->fd_buffered, &st) != 0) {
+        int64_t e = -(int64_t)errno;
+        release_file(*f);
+        return e;
+    }
+    f->size = (uint64_t)st.st_size;
+    if (mode != FSTX_READ_BUFFERED) {
+        f->fd_direct = open(path, O_RDONLY | O_CLOEXEC | O_DIRECT); // EINVAL on some filesystems
+        if (f->fd_direct < 0) fstx_internal::debug("file_open: no O_DIRECT for %s (%s)", path, std::strerror(errno));
+    }
+    if (mode == FSTX_READ_AUTO && f->fd_direct >= 0 && f->size > 0) {
+        void *m = mmap(nullptr, f->size, PROT_READ, MAP_SHARED, f->fd_buffered, 0);
+        if (m != MAP_FAILED) f->map = m;
+    }
+    std::lock_guard<std::mutex> lk(ctx->table_mutex);
+    int64_t id = ctx->next_file++;
+    ctx->files[id] = f;
+    return id;
+}
+
+int fstx_file_close(fstx_ctx *ctx, int64_t file) {
+    if (!ctx) return -FSTX_E_INVAL;
+    std::shared_ptr<FileEntry> f;
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        auto it = ctx->files.find(file);
+        if (it == ctx->files.end()) return -FSTX_E_NO_REQ;
+        if (it->second->open_requests.load() != 0) return -EBUSY;
+        f = it->second;
+        ctx->files.erase(it);
+    }
+    release_file(*f);
+    return 0;
+}
+
+// ---- requests ------------------------------------------------------------------
+
+int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_t length,
+                         void *dev_base, uint64_t dev_capacity, uint64_t dst_off) {
+    if (!ctx || (!dev_base && length)) return -FSTX_E_INVAL;
+    if (dst_off > dev_capacity || length > dev_capacity - dst_off) return -FSTX_E_RANGE;
+    auto req = std::make_shared<Request>();
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        auto it = ctx->files.find(file);
+        if (it == ctx->files.end()) return -FSTX_E_NO_REQ;
+        req->file = it->second;
+        req->id = ctx->next_request++;
+        ctx->requests[req->id] = req;
+        req->file->open_requests.fetch_add(1);
+    }
+    req->length = length;
+    if (file_off > req->file->size || length > req->file->size - file_off)
+        req->error.store(-FSTX_E_SHORT_READ); // reported by wait_read, like a failed read
+
+    // Cut on multiples of block_bytes counted from the 4 KiB boundary below the
+    // first byte, so that every block's O_DIRECT window fits one slot.
+    std::vector<Block> blocks;
+    if (length && req->error.load() == 0) {
+        const uint64_t bb = ctx->cfg.block_bytes;
+        const uint64_t origin = align_down(file_off, kPage);
+        const uint64_t end = file_off + length;
+        for (uint64_t lo = origin; lo < end; lo += bb) {
+            uint64_t a = std::max(lo, file_off), z = std::min(lo + bb, end);
+            blocks.push_back(Block{req, a, z - a, static_cast<char *>(dev_base) + dst_off + (a - file_off)});
+        }
+    }
+    req->blocks_left.store(blocks.size());
+    if (!blocks.empty()) {
+        {
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+            if (ctx->closing) {
+                std::lock_guard<std::mutex> lk2(ctx->table_mutex);
+                ctx->requests.erase(req->id);
+                req->file->open_requests.fetch_sub(1);
+                return -FSTX_E_CLOSED;
+            }
+            for (Block &b : blocks) ctx->queue.push_back(std::move(b));
+        }
+        ctx->q_cv.notify_all();
+    }
+    return req->id;
+}
+
+int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request) {
+    if (!ctx) return -FSTX_E_INVAL;
+    std::shared_ptr<Request> req;
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        auto it = ctx->requests.find(request);
+        if (it == ctx->requests.end()) return -FSTX_E_NO_REQ;
+        req = it->second;
+        ctx->requests.erase(it);
+    }
+    {
+        std::unique_lock<std::mutex> lk(ctx->done_mutex);
+        ctx->done_cv.wait(lk, [&] { return req->blocks_left.load(std::memory_order_acquire) == 0; });
+    }
+    // every block is enqueued on its stream by now; wait for the copies themselves
+    int64_t status = req->error.load();
+    uint64_t mask = req->stream_mask.load();
+    fstx_dev::set_device(ctx->cfg.device_id);
+    for (size_t i = 0; i < ctx->streams.size(); ++i)
+        if (mask & (1ull << i)) {
+            int rc = fstx_dev::stream_sync(ctx->streams[i]);
+            if (rc < 0 && status == 0) status = rc;
+        }
+    req->file->open_requests.fetch_sub(1);
+    return status < 0 ? status : (int64_t)req->length;
+}
+
+int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
+    if (!ctx || !out) return -FSTX_E_INVAL;
+    const Counters &c = ctx->ctr;
+    out->bounce_buffer_bytes = ctx->ring_bytes;
+    out->bytes_read = c.bytes_read.load();
+    out->bytes_copied = c.bytes_copied.load();
+    out->blocks_buffered = c.blocks_buffered.load();
+    out->blocks_direct = c.blocks_direct.load();
+    out->read_ns = c.read_ns.load();
+    out->stage_ns = c.stage_ns.load();
+    out->slot_wait_ns = c.slot_wait_ns.load();
+    out->direct_fallbacks = c.direct_fallbacks.load();
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,162 @@
+# SPDX-License-Identifier: Apache-2.0
+"""Framework abstraction of the load path.
+
+Same contract as the reference's ``fastsafetensors/frameworks/__init__.py``:
+``TensorBase`` (``:11-62``), ``ProcessGroupBase`` (``:67-105``) and
+``FrameworkOpBase`` (``:111-253``).  Only the PyTorch backend exists here; the
+two members that are new (``view_tensor`` and ``extract_shard``) are where this
+package hands work to its HIP library instead of DLPack capsules and
+``Tensor.contiguous()``.
+"""
+
+from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import Any, List, Optional, Sequence, Tuple
+
+from ..st_types import Device, DType
+
+
+@dataclass
+class TensorBase(ABC):
+    device: Device
+    dtype: DType
+
+    @abstractmethod
+    def get_raw(self) -> Any: ...
+
+    @abstractmethod
+    def contiguous(self) -> "TensorBase": ...
+
+    @abstractmethod
+    def to(self, device: Optional[Device] = None, dtype: DType = DType.AUTO) -> "TensorBase": ...
+
+    @abstractmethod
+    def clone(self) -> "TensorBase": ...
+
+    @abstractmethod
+    def detach(self) -> "TensorBase": ...
+
+    @abstractmethod
+    def view(self, dtype: DType) -> "TensorBase": ...
+
+    @abstractmethod
+    def __getitem__(self, index) -> "TensorBase": ...
+
+    def reshape(self, shape: List[int]) -> "TensorBase":
+        raise NotImplementedError(f"{type(self).__name__} does not implement reshape()")
+
+    def data_ptr(self) -> int:
+        raise NotImplementedError(f"{type(self).__name__} does not implement data_ptr()")
+
+
+class ProcessGroupBase(ABC):
+    """The six operations the load path needs from a process group."""
+
+    @abstractmethod
+    def size(self) -> int: ...
+
+    @abstractmethod
+    def rank(self) -> int: ...
+
+    @abstractmethod
+    def broadcast(self, dst: TensorBase, rank: int) -> None: ...
+
+    @abstractmethod
+    def scatter(self, dst: TensorBase, scatter_list: List[TensorBase], src: int) -> None: ...
+
+    @abstractmethod
+    def send(self, t: TensorBase, dst_rank: int, tag: int) -> None: ...
+
+    @abstractmethod
+    def recv(self, t: TensorBase, src_rank: int, tag: int) -> None: ...
+
+
+class FrameworkOpBase(ABC):
+    @abstractmethod
+    def get_name(self) -> str: ...
+
+    @abstractmethod
+    def get_device(self, device: str, pg: ProcessGroupBase) -> Device: ...
+
+    @abstractmethod
+    def set_device(self, device: Device) -> None: ...
+
+    @abstractmethod
+    def alloc_tensor_memory(self, length: int, dev: Device) -> Any: ...
+
+    @abstractmethod
+    def free_tensor_memory(self, gbuf: Any, dev: Device) -> None: ...
+
+    @abstractmethod
+    def get_empty_tensor(self, shape: List[int], dtype: DType, device: Device) -> TensorBase: ...
+
+    @abstractmethod
+    def concat_tensors(self, tensors: List[TensorBase], dim: int) -> TensorBase: ...
+
+    @abstractmethod
+    def copy_tensor(self, dst: TensorBase, src: TensorBase) -> None: ...
+
+    @abstractmethod
+    def get_dtype_size(self, dtype: DType) -> float: ...
+
+    @abstractmethod
+    def get_cuda_ver(self) -> str: ...
+
+    @abstractmethod
+    def get_device_ptr_align(self) -> int: ...
+
+    @abstractmethod
+    def as_workaround_dtype(self, dtype: DType) -> DType: ...
+
+    @abstractmethod
+    def view_tensor(self, gbuf: Any, byte_offset: int, frame: Any, device: Device) -> TensorBase:
+        """Zero-copy tensor over ``gbuf[byte_offset : byte_offset + frame.nbytes]``."""
+
+    @abstractmethod
+    def extract_shard(
+        self, src: TensorBase, frame: Any, dim: int, rank: int, world: int
+    ) -> TensorBase:
+        """Dense copy of rank ``rank``'s ``ceil(S/world)`` block of ``src`` along ``dim``."""
+
+    def get_storage_shape(
+        self, dtype: DType, shape: List[int], strides: List[int]
+    ) -> Tuple[List[int], List[int]]:
+        return shape, strides
+
+    def get_native_shape(self, dtype: DType, st_shape: List[int]) -> List[int]:
+        return st_shape
+
+    def get_native_slices(self, dtype: DType, st_shape: Sequence[int], slices: Tuple) -> Tuple:
+        return slices
+
+    def synchronize(self, device: Device) -> None:
+        return None
+
+    def get_global_rank(self) -> int:
+        return 0
+
+    def get_device_name(self, index: int) -> str:
+        return ""
+
+    @abstractmethod
+    def get_process_group(self, pg: Optional[Any]) -> ProcessGroupBase: ...
+
+    @abstractmethod
+    def is_equal(self, wrapped: TensorBase, real: Any) -> bool: ...
+
+    @abstractmethod
+    def randn(self, s: tuple, device: Device, dtype: DType) -> TensorBase: ...
+
+    @abstractmethod
+    def support_fp8(self) -> bool: ...
+
+    @abstractmethod
+    def get_mem_used(self) -> int: ...
+
+
+def get_framework_op(name: str) -> FrameworkOpBase:
+    if name in ("pt", "pytorch", "torch"):
+        from ._torch import get_framework_op as make
+
+        return make()
+    raise Exception(f"Unknown framework name: {name}")

@@ -1,0 +1,372 @@
+# SPDX-License-Identifier: Apache-2.0
+"""PyTorch-ROCm backend of the framework abstraction.
+
+Counterpart of the reference's ``fastsafetensors/frameworks/_torch.py``:
+dtype table (``:17-49``), tensor wrapper (``:52-98``), process group wrapper
+(``:125-225``) and ``TorchOp`` (``:228-452``).  Differences that matter:
+
+* device memory of a file is one ``torch.uint8`` tensor from torch's caching
+  allocator and tensors are ``view``s of slices of it, instead of raw
+  ``caching_allocator_alloc`` pointers wrapped in DLPack capsules
+  (``_torch.py:243-257``, ``dlpack.py:240-247``);
+* a rank's shard is produced by the slice-extract kernel of ``libfstx``
+  (``extract_shard``), not by ``Tensor.contiguous()``;
+* one GPU only: the process group is either a world of one or a
+  ``StubProcessGroup(rank, size)`` that *reports* rank r of N so that the
+  shard of any tensor-parallel rank can be produced on this GPU.  A real
+  ``torch.distributed`` group is rejected.
+"""
+
+import math
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import _native
+from ..common import SingleGroup, TensorFrame
+from ..st_types import Device, DeviceType, DType, dtype_size
+from . import FrameworkOpBase, ProcessGroupBase, TensorBase
+
+dtype_convert: Dict[DType, torch.dtype] = {
+    DType.BOOL: torch.bool,
+    DType.U8: torch.uint8,
+    DType.I8: torch.int8,
+    DType.I16: torch.int16,
+    DType.I32: torch.int32,
+    DType.I64: torch.int64,
+    DType.U16: torch.uint16,
+    DType.U32: torch.uint32,
+    DType.U64: torch.uint64,
+    DType.F16: torch.float16,
+    DType.BF16: torch.bfloat16,
+    DType.F32: torch.float32,
+    DType.F64: torch.float64,
+    DType.F8_E5M2: torch.float8_e5m2,
+    DType.F8_E4M3: torch.float8_e4m3fn,
+    DType.F8_E8M0: torch.float8_e8m0fnu,
+    DType.F4: torch.float4_e2m1fn_x2,
+}
+# dtypes the reference routes through an integer view before DLPack (``_torch.py:29-34``)
+need_workaround_dtypes: Dict[DType, DType] = {
+    DType.F8_E5M2: DType.I8,
+    DType.F8_E4M3: DType.I8,
+    DType.F8_E8M0: DType.U8,
+    DType.F4: DType.U8,
+}
+
+
+@dataclass
+class TorchTensor(TensorBase):
+    real_tensor: torch.Tensor
+
+    def _wrap(self, t: torch.Tensor) -> "TorchTensor":
+        return TorchTensor(self.device, self.dtype, t)
+
+    def get_raw(self) -> torch.Tensor:
+        return self.real_tensor
+
+    def contiguous(self) -> "TorchTensor":
+        return self._wrap(self.real_tensor.contiguous())
+
+    def to(self, device: Optional[Device] = None, dtype: DType = DType.AUTO) -> "TorchTensor":
+        move = device is not None and device != self.device
+        cast = dtype not in (DType.AUTO, self.dtype)
+        if not (move or cast):
+            return self
+        t = self.real_tensor.to(
+            device=device.as_str() if move else None, dtype=dtype_convert[dtype] if cast else None
+        )
+        return TorchTensor(device if move else self.device, dtype if cast else self.dtype, t)
+
+    def clone(self) -> "TorchTensor":
+        return self._wrap(self.real_tensor.clone())
+
+    def detach(self) -> "TorchTensor":
+        return self._wrap(self.real_tensor.detach())
+
+    def view(self, dtype: DType) -> "TorchTensor":
+        return TorchTensor(self.device, dtype, self.real_tensor.view(dtype_convert[dtype]))
+
+    def __getitem__(self, index) -> "TorchTensor":
+        return self._wrap(self.real_tensor[index])
+
+    def reshape(self, shape: List[int]) -> "TorchTensor":
+        return self._wrap(self.real_tensor.reshape(shape))
+
+    def data_ptr(self) -> int:
+        return self.real_tensor.data_ptr()
+
+
+class TorchProcessGroup(ProcessGroupBase):
+    """World of one process: every exchange is the identity."""
+
+    def size(self) -> int:
+        return 1
+
+    def rank(self) -> int:
+        return 0
+
+    def broadcast(self, dst: TorchTensor, rank: int) -> None:
+        return None
+
+    def scatter(self, dst: TorchTensor, scatter_list: List[TorchTensor], src: int) -> None:
+        return None
+
+    def send(self, t: TorchTensor, dst_rank: int, tag: int) -> None:
+        return None
+
+    def recv(self, t: TorchTensor, src_rank: int, tag: int) -> None:
+        return None
+
+
+class StubProcessGroup(TorchProcessGroup):
+    """Reports ``rank`` of ``size`` without any peer.
+
+    ``get_sharded`` then returns exactly the block that rank would receive from
+    the owner's scatter, computed on this GPU.  ``scatter`` keeps that meaning
+    for callers that hand it a full list: element ``rank`` lands in ``dst``.
+    ``send``/``recv`` have no peer to talk to and leave their tensors untouched.
+    """
+
+    def __init__(self, rank: int, size: int):
+        if size < 1 or not 0 <= rank < size:
+            raise ValueError(f"StubProcessGroup: rank {rank} is outside a world of {size}")
+        self._rank, self._size = rank, size
+
+    def size(self) -> int:
+        return self._size
+
+    def rank(self) -> int:
+        return self._rank
+
+    def scatter(self, dst: TorchTensor, scatter_list: List[TorchTensor], src: int) -> None:
+        if scatter_list:
+            dst.real_tensor.copy_(scatter_list[self._rank].real_tensor)
+
+
+class TorchOp(FrameworkOpBase):
+    def __init__(self) -> None:
+        self.mem_used = 0
+
+    def get_name(self) -> str:
+        return "pytorch"
+
+    def get_device(self, device: str, pg: ProcessGroupBase) -> Device:
+        dev = torch.device(device)
+        return Device(DeviceType(dev.type), dev.index)
+
+    def set_device(self, device: Device) -> None:
+        if device.type != DeviceType.CPU:
+            torch.cuda.set_device(device.as_str())
+
+    # ---- memory ------------------------------------------------------------
+    def alloc_tensor_memory(self, length: int, dev: Device) -> _native.DeviceBuffer:
+        arena = torch.empty(max(length, 1), dtype=torch.uint8, device=dev.as_str())
+        self.mem_used += length
+        return _native.DeviceBuffer(arena.data_ptr(), length, dev.type != DeviceType.CPU, arena)
+
+    def free_tensor_memory(self, gbuf: _native.DeviceBuffer, dev: Device) -> None:
+        self.mem_used -= gbuf.total_length()
+        gbuf.extras.clear()
+        gbuf.keepalive = None
+
+    def shrink_tensor_memory(self, gbuf: _native.DeviceBuffer) -> None:
+        """Give back the main allocation of ``gbuf`` but keep its side allocations."""
+        self.mem_used -= gbuf.get_length()
+        gbuf.keepalive = None
+        gbuf._base, gbuf._length = 0, 0
+
+    def alloc_side_memory(self, gbuf: _native.DeviceBuffer, length: int, dev: Device) -> _native.DeviceBuffer:
+        """Allocation that lives and dies with ``gbuf`` (counted in ``mem_used``)."""
+        side = self.alloc_tensor_memory(length, dev)
+        gbuf.extras.append(side)
+        return side
+
+    def get_empty_tensor(self, shape: List[int], dtype: DType, device: Device) -> TorchTensor:
+        t = torch.empty(
+            self.get_native_shape(dtype, shape), dtype=dtype_convert[dtype], device=device.as_str()
+        )
+        return TorchTensor(device, dtype, t)
+
+    def view_tensor(
+        self, gbuf: _native.DeviceBuffer, byte_offset: int, frame: TensorFrame, device: Device
+    ) -> TorchTensor:
+        nbytes = frame.nbytes
+        if byte_offset < 0 or byte_offset + nbytes > gbuf.get_length():
+            raise IndexError(
+                f"out of bound access: length={gbuf.get_length()}, request offset={byte_offset}, "
+                f"request length={nbytes}"
+            )
+        raw = gbuf.keepalive[byte_offset : byte_offset + nbytes]
+        t = raw.view(dtype_convert[frame.dtype]).view(self.get_native_shape(frame.dtype, frame.shape))
+        return TorchTensor(device, frame.dtype, t)
+
+    def concat_tensors(self, tensors: List[TorchTensor], dim: int) -> TorchTensor:
+        first = tensors[0]
+        if first.dtype in (DType.F8_E8M0, DType.F4):
+            joined = torch.cat([t.real_tensor.view(torch.uint8) for t in tensors], dim=dim)
+            return TorchTensor(first.device, first.dtype, joined.view(dtype_convert[first.dtype]))
+        return TorchTensor(first.device, first.dtype, torch.cat([t.real_tensor for t in tensors], dim=dim))
+
+    def copy_tensor(self, dst: TorchTensor, src: TorchTensor) -> None:
+        dst.real_tensor.copy_(src.real_tensor)
+
+    # ---- dtype facts ---------------------------------------------------------
+    def get_dtype_size(self, dtype: DType) -> float:
+        return dtype_size(dtype)
+
+    def get_cuda_ver(self) -> str:
+        if not torch.cuda.is_available():
+            return "0.0"
+        if getattr(torch.version, "hip", None):
+            return f"hip-{torch.version.hip}"
+        return f"cuda-{torch.version.cuda}"
+
+    def get_device_ptr_align(self) -> int:
+        return 16
+
+    def as_workaround_dtype(self, dtype: DType) -> DType:
+        return need_workaround_dtypes.get(dtype, dtype)
+
+    def _pack_ratio(self, dtype: DType, shape: Sequence[int]) -> int:
+        """Logical elements per storage byte (2 for F4, else 1); validates the last dim."""
+        size = dtype_size(dtype)
+        if size >= 1.0:
+            return 1
+        ratio = round(1.0 / size)
+        if not shape or shape[-1] % ratio:
+            raise ValueError(
+                f"Malformed input: shape={list(shape)}, ratio={ratio}, "
+                "last dimension must be divisible by the packing ratio."
+            )
+        return ratio
+
+    def get_storage_shape(
+        self, dtype: DType, shape: List[int], strides: List[int]
+    ) -> Tuple[List[int], List[int]]:
+        ratio = self._pack_ratio(dtype, shape)
+        if ratio == 1:
+            return shape, strides
+        return [math.prod(shape) // ratio], [1]
+
+    def get_native_shape(self, dtype: DType, st_shape: List[int]) -> List[int]:
+        ratio = self._pack_ratio(dtype, st_shape)
+        if ratio == 1:
+            return st_shape
+        return list(st_shape[:-1]) + [st_shape[-1] // ratio]
+
+    def get_native_slices(self, dtype: DType, st_shape: Sequence[int], slices: Tuple) -> Tuple:
+        if dtype_size(dtype) >= 1.0 or not st_shape or len(slices) < len(st_shape):
+            return slices
+        ratio = round(1.0 / dtype_size(dtype))
+        extent = st_shape[-1]
+        last = slices[-1]
+
+        def packed(v: int, what: str) -> int:
+            if v % ratio:
+                raise ValueError(
+                    f"Malformed input: slices={slices}, ratio={ratio}, packed sub-byte {what} "
+                    "must align to storage units."
+                )
+            return v // ratio
+
+        if isinstance(last, slice):
+            if last.step not in (None, 1):
+                raise ValueError(
+                    f"Malformed input: slices={slices}, ratio={ratio}, "
+                    "packed sub-byte slices only support step=1."
+                )
+            lo = min(max(0 if last.start is None else last.start, 0), extent)
+            hi = min(max(extent if last.stop is None else last.stop, 0), extent)
+            last = slice(packed(lo, "slice bounds"), packed(hi, "slice bounds"), 1 if last.step is None else last.step)
+        elif isinstance(last, int):
+            last = packed(last, "indices")
+        return tuple(slices[:-1]) + (last,)
+
+    # ---- shard extraction ----------------------------------------------------
+    def shard_geometry(self, frame: TensorFrame, dim: int, rank: int, world: int) -> Tuple[List[int], int, int, int, int]:
+        """Shape and copy geometry of rank ``rank``'s block of ``frame`` along ``dim``.
+
+        Returns ``(shard_shape, outer, seg_bytes, src_pitch, src_byte_offset)`` in
+        terms of the tensor's row-major bytes: ``outer`` segments of
+        ``seg_bytes``, ``src_pitch`` apart, the first at ``src_byte_offset``.
+        """
+        shape = frame.shape
+        if not 0 <= dim < len(shape):
+            raise IndexError(f"shard dim {dim} is outside shape {shape}")
+        extent = shape[dim]
+        block = -(-extent // world)
+        lo = min(rank * block, extent)
+        hi = min(lo + block, extent)
+        bits = int(dtype_size(frame.dtype) * 8)
+        inner_bits = math.prod(shape[dim + 1 :]) * bits
+        if (inner_bits * lo) % 8 or (inner_bits * hi) % 8 or (inner_bits * extent) % 8:
+            raise ValueError(
+                f"Malformed input: shape={shape}, dim={dim}, packed sub-byte slice bounds must "
+                "align to storage units."
+            )
+        outer = math.prod(shape[:dim])
+        out_shape = list(shape)
+        out_shape[dim] = hi - lo
+        return out_shape, outer, inner_bits * (hi - lo) // 8, inner_bits * extent // 8, inner_bits * lo // 8
+
+    def extract_shard(self, src: TorchTensor, frame: TensorFrame, dim: int, rank: int, world: int) -> TorchTensor:
+        out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world)
+        dst = self.get_empty_tensor(out_shape, frame.dtype, src.device)
+        if outer * seg:
+            if not src.real_tensor.is_cuda:
+                raise RuntimeError("extract_shard needs a tensor in GPU memory (no CPU path exists)")
+            stream = torch.cuda.current_stream(src.real_tensor.device).cuda_stream
+            _native.slice_copy(dst.data_ptr(), src.data_ptr() + first, outer, seg, pitch, stream)
+        return dst
+
+    # ---- misc ------------------------------------------------------------------
+    def synchronize(self, device: Device) -> None:
+        if device.type != DeviceType.CPU and torch.cuda.is_available():
+            torch.cuda.synchronize()
+
+    def get_device_name(self, index: int) -> str:
+        try:
+            return torch.cuda.get_device_name(index) if torch.cuda.is_available() else ""
+        except Exception:
+            return ""
+
+    def get_process_group(self, pg: Optional[Any]) -> ProcessGroupBase:
+        if pg is None or isinstance(pg, SingleGroup):
+            return TorchProcessGroup()
+        if isinstance(pg, ProcessGroupBase):
+            return pg
+        raise Exception(
+            "pg must be None, SingleGroup or StubProcessGroup: this loader drives one GPU and "
+            "has no torch.distributed exchange"
+        )
+
+    def is_equal(self, wrapped: TorchTensor, real: Any) -> bool:
+        if not isinstance(real, torch.Tensor):
+            raise Exception("real is not torch.Tensor")
+        a, b = wrapped.real_tensor, real
+        if a.shape != b.shape or a.dtype != b.dtype:
+            return False
+        if a.dtype in (torch.float8_e8m0fnu, torch.float4_e2m1fn_x2):
+            a, b = a.view(torch.uint8), b.view(torch.uint8)
+        return bool(torch.all(a.eq(b)))
+
+    def randn(self, s: tuple, device: Device, dtype: DType) -> TorchTensor:
+        return TorchTensor(device, dtype, torch.randn(s, device=device.as_str(), dtype=dtype_convert[dtype]))
+
+    def support_fp8(self) -> bool:
+        return True
+
+    def get_mem_used(self) -> int:
+        return self.mem_used
+
+
+_op: Optional[TorchOp] = None
+
+
+def get_framework_op() -> TorchOp:
+    global _op
+    if _op is None:
+        _op = TorchOp()
+    return _op

@@ -1,0 +1,196 @@
+/* SPDX-License-Identifier: Apache-2.0
+ *
+ * fstx: C ABI of the MI355X safetensors load path.
+ *
+ * One shared library (libfstx.so, HIP, gfx950) holds
+ *   - the file -> pinned ring -> HBM copy pipeline, and
+ *   - the two data-movement kernels that post-process tensors in HBM
+ *     (realign copy, slice extract).
+ * Every entry point takes plain pointers and sizes; there are no C++ or torch
+ * types in the signatures, so the library binds from ctypes, cgo, JNI or any
+ * other FFI.  Each declaration names the interface of the reference
+ * (foundation-model-stack/fastsafetensors 0.3.2, paths relative to its root)
+ * that it stands in for.
+ *
+ * Conventions
+ *   - int / int64_t returns: >= 0 success, < 0 is -(fstx_status) or -errno
+ *     (errno values are < FSTX_E_BASE in magnitude); never aborts, never
+ *     prints unless fstx_set_debug_log(1).
+ *   - `stream` is a hipStream_t passed as void*; NULL is the device's null
+ *     stream.  Kernel entry points only enqueue work; they do not synchronize.
+ *   - Device pointers must belong to the device that is current on the
+ *     calling thread (kernels) or to the context's device (reads).
+ */
+#ifndef FSTX_H
+#define FSTX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSTX_ABI_VERSION 1
+
+/* status codes beyond errno */
+#define FSTX_E_BASE 10000
+enum fstx_status {
+    FSTX_OK = 0,
+    FSTX_E_INVAL = FSTX_E_BASE + 1,     /* bad argument                                 */
+    FSTX_E_HIP = FSTX_E_BASE + 2,       /* a HIP runtime call failed                    */
+    FSTX_E_RANGE = FSTX_E_BASE + 3,     /* destination range exceeds the device buffer  */
+    FSTX_E_SHORT_READ = FSTX_E_BASE + 4,/* file ended before the requested range        */
+    FSTX_E_NO_REQ = FSTX_E_BASE + 5,    /* unknown or already-waited request id         */
+    FSTX_E_CLOSED = FSTX_E_BASE + 6,    /* context is shutting down                     */
+    FSTX_E_NO_DEVICE = FSTX_E_BASE + 7, /* no HIP device visible                        */
+    FSTX_E_TOO_MANY = FSTX_E_BASE + 8   /* batch larger than FSTX_BATCH_MAX             */
+};
+
+/* read modes of fstx_file_open / fstx_submit_read */
+enum fstx_read_mode {
+    FSTX_READ_AUTO = 0,     /* per block: buffered when the block is in the page cache, else O_DIRECT */
+    FSTX_READ_BUFFERED = 1, /* page-cache pread straight into the pinned ring                         */
+    FSTX_READ_DIRECT = 2    /* O_DIRECT pread into an aligned staging block, then into the ring       */
+};
+
+typedef struct fstx_ctx fstx_ctx;
+
+typedef struct fstx_config {
+    uint32_t struct_size;    /* = sizeof(fstx_config); lets the struct grow                      */
+    int32_t device_id;       /* HIP device ordinal                                               */
+    int32_t numa_node;       /* node to pin I/O threads and the ring to; < 0 = do not pin        */
+    uint32_t n_threads;      /* I/O worker threads (0 = default 8)                               */
+    uint32_t n_streams;      /* HIP copy streams shared by the workers (0 = default 4)           */
+    uint64_t block_bytes;    /* bytes per read block = per ring slot, multiple of 4096 (0 = 4 MiB)*/
+    uint32_t slots_per_thread; /* ring slots each worker cycles through (0 = default 2)          */
+    uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 4)      */
+} fstx_config;
+
+typedef struct fstx_metrics {
+    uint64_t bounce_buffer_bytes; /* pinned ring bytes currently allocated by this context       */
+    uint64_t bytes_read;          /* file bytes delivered into the ring                          */
+    uint64_t bytes_copied;        /* bytes enqueued host -> device                               */
+    uint64_t blocks_buffered;     /* blocks served by page-cache pread                           */
+    uint64_t blocks_direct;       /* blocks served by O_DIRECT                                   */
+    uint64_t read_ns;             /* summed over workers: time inside pread                      */
+    uint64_t stage_ns;            /* summed over workers: staging memcpy after O_DIRECT          */
+    uint64_t slot_wait_ns;        /* summed over workers: waiting for a ring slot's last copy    */
+    uint64_t direct_fallbacks;    /* blocks that asked for O_DIRECT but were read buffered       */
+} fstx_metrics;
+
+/* ---- library-wide helpers ------------------------------------------------ */
+
+/* ABI version of the loaded library (FSTX_ABI_VERSION). */
+int fstx_abi_version(void);
+
+/* Number of visible HIP devices, or -FSTX_E_NO_DEVICE.
+ * Stands in for load_library_functions + is_hip_found (cpp/ext.cpp:278-410). */
+int fstx_device_count(void);
+
+/* Required alignment of O_DIRECT windows: 4096.  get_alignment_size (cpp/ext.cpp:412-415). */
+int fstx_get_alignment_size(void);
+
+/* "dddd:bb:dd.f" PCI id of a device into out[len].  get_device_pci_bus (cpp/ext.cpp:508-523). */
+int fstx_get_device_pci_bus(int device_id, char *out, int len);
+
+/* Restrict the calling thread (and threads it creates later) to the CPUs of a
+ * NUMA node and prefer its memory.  set_numa_node (cpp/ext.cpp:525-533). */
+int fstx_set_numa_node(int numa_node);
+
+/* Toggle debug lines on stderr.  set_debug_log (cpp/ext.cpp:417-420). */
+void fstx_set_debug_log(int enabled);
+
+/* Pinned ring bytes alive in the whole process.
+ * get_cpp_metrics().bounce_buffer_bytes (cpp/ext.cpp:952-954). */
+uint64_t fstx_bounce_buffer_bytes(void);
+
+/* Text for a negative return value (errno or fstx_status); never NULL. */
+const char *fstx_strerror(int64_t code);
+
+/* 4096-aligned host allocation.  cpu_malloc / cpu_free (cpp/ext.cpp:542-557). */
+void *fstx_host_alloc(uint64_t length);
+void fstx_host_free(void *p);
+
+/* ---- file -> HBM pipeline -------------------------------------------------- */
+
+/* Create the reader: worker threads, copy streams and the pinned ring
+ * (allocated once, reused by every file).  Replaces the nogds_file_reader
+ * constructor (cpp/ext.hpp:176-180) and its lazy cudaHostAlloc (cpp/ext.cpp:735-751). */
+int fstx_ctx_create(const fstx_config *cfg, fstx_ctx **out);
+
+/* Drain outstanding work, join the workers, free ring, streams and events.
+ * ~nogds_file_reader (cpp/ext.cpp:778-806). */
+int fstx_ctx_destroy(fstx_ctx *ctx);
+
+/* Open a file for reading in `mode`; returns a file handle >= 1.
+ * The reference's Python opens the fd itself (copier/nogds.py:26-31); here the
+ * library owns the descriptors because O_DIRECT needs its own. */
+int64_t fstx_file_open(fstx_ctx *ctx, const char *path, int mode);
+
+/* Close a handle; outstanding requests on it must have been waited. */
+int fstx_file_close(fstx_ctx *ctx, int64_t file);
+
+/* Enqueue: copy file bytes [file_off, file_off+length) to dev_base + dst_off.
+ * dev_capacity is the size of the device buffer at dev_base; the range is
+ * checked against it (gds_device_buffer::_get_raw_pointer, cpp/ext.hpp:139-146).
+ * Returns a request id >= 1 immediately; I/O proceeds on the workers.
+ * nogds_file_reader::submit_read (cpp/ext.cpp:726-763). */
+int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_t length,
+                         void *dev_base, uint64_t dev_capacity, uint64_t dst_off);
+
+/* Block until every byte of the request is in device memory; returns the byte
+ * count or a negative error.  The id is consumed.
+ * nogds_file_reader::wait_read (cpp/ext.cpp:765-776). */
+int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request);
+
+/* Snapshot of the context's counters. */
+int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out);
+
+/* ---- HBM kernels ----------------------------------------------------------- */
+
+/* dst[0:nbytes) = src[0:nbytes), any byte alignment on either side, ranges
+ * must not overlap.  The bulk moves as 16-byte vectors with the source
+ * funnel-shifted into place.  Replaces gds_device_buffer::memmove
+ * (cpp/ext.cpp:606-645), which the reference drives to shift a file's data
+ * section down by header_length % 16 bytes (copier/gds.py:138-159). */
+int fstx_realign_copy(void *dst, const void *src, uint64_t nbytes, void *stream);
+
+typedef struct fstx_copy_desc {
+    void *dst;
+    const void *src;
+    uint64_t nbytes;
+} fstx_copy_desc;
+
+#define FSTX_BATCH_MAX 48
+
+/* n <= FSTX_BATCH_MAX independent realign copies in one launch. */
+int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, void *stream);
+
+/* Gather `outer` segments of seg_bytes, the o-th read from src + o*src_pitch,
+ * into dst + o*seg_bytes (a dense [outer, seg_bytes] block).  This is one
+ * rank's shard of a row-major tensor cut along a dimension: for shape
+ * [.., S, ..] cut at dim d into blocks of bs, outer = prod(shape[:d]),
+ * src_pitch = S * inner_bytes, seg_bytes = rows_of_this_rank * inner_bytes and
+ * src already points at the rank's first row.  Replaces the per-rank
+ * t[slices].contiguous() of LazyTensorFactory.shuffle (tensor_factory.py:168-175). */
+int fstx_slice_copy(void *dst, const void *src, uint64_t outer, uint64_t seg_bytes,
+                    uint64_t src_pitch, void *stream);
+
+typedef struct fstx_slice_desc {
+    void *dst;
+    const void *src;
+    uint64_t outer;
+    uint64_t seg_bytes;
+    uint64_t src_pitch;
+} fstx_slice_desc;
+
+/* n <= FSTX_BATCH_MAX slice extractions in one launch (the shards of many
+ * tensors for one rank, as FilesBufferOnDevice.as_dict asks for them,
+ * file_buffer.py:238-259). */
+int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSTX_H */
