@@ -1,0 +1,199 @@
+# SPDX-License-Identifier: Apache-2.0
+"""GPU parity of the two HBM kernels, called through the C ABI, against the CPU oracle.
+
+Bit-exact is the bar (pure byte movement).  Device memory and streams come from
+torch; the kernels are libfstx's.
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from fastsafetensors_amd import _native
+from oracle import st_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    assert _native.device_count() > 0
+    return torch.device("cuda:0")
+
+
+def stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def rand_bytes(n: int, seed: int) -> np.ndarray:
+    return np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8)
+
+
+def to_dev(a: np.ndarray, dev, pad: int = 64) -> torch.Tensor:
+    """Device copy of ``a`` with ``pad`` guard bytes on both sides (value 0xA5)."""
+    host = np.full(a.size + 2 * pad, 0xA5, dtype=np.uint8)
+    host[pad : pad + a.size] = a
+    return torch.from_numpy(host).to(dev)
+
+
+# ---- realign copy -------------------------------------------------------------------------
+
+SIZES = [0, 1, 2, 15, 16, 17, 31, 33, 255, 256, 4095, 4096, 4097, 65536 + 5, (1 << 20) + 3]
+
+
+def test_realign_all_alignments(dev):
+    """Every (src % 16, dst % 16) pair at sizes around the 16-byte and 4 KiB edges;
+    guard bytes around the destination must stay untouched."""
+    src_host = rand_bytes((1 << 20) + 256, 1)
+    src = torch.from_numpy(src_host).to(dev)
+    for n in SIZES:
+        dst = torch.full((n + 256,), 0xA5, dtype=torch.uint8, device=dev)
+        for so, do in itertools.product(range(16), range(16)):
+            if n > 70000 and (so * 16 + do) % 37:  # thin out the big sizes
+                continue
+            dst.fill_(0xA5)
+            _native.realign_copy(dst.data_ptr() + 64 + do, src.data_ptr() + so, n, stream())
+            got = dst.cpu().numpy()
+            assert np.array_equal(got[64 + do : 64 + do + n], src_host[so : so + n]), (n, so, do)
+            assert (got[: 64 + do] == 0xA5).all() and (got[64 + do + n :] == 0xA5).all(), (n, so, do)
+
+
+def test_realign_matches_reference_memmove_semantics(dev):
+    """Shifting a window down by header_length % 16, as copier/gds.py:138-159 does
+    through a temporary: compare with the oracle's memmove."""
+    for header_length in (104, 4096 + 2, 8192 + 10, 12288 + 15):
+        lead = header_length % 4096
+        window = rand_bytes(lead + 300_001, header_length)
+        want = orc.realign(window, header_length, header_length - lead, 300_001)
+        w = torch.from_numpy(window).to(dev)
+        out = torch.empty(300_001, dtype=torch.uint8, device=dev)
+        _native.realign_copy(out.data_ptr(), w.data_ptr() + lead, 300_001, stream())
+        assert np.array_equal(out.cpu().numpy(), want)
+        # DeviceBuffer.memmove (two copies through tmp) gives the same bytes in place
+        buf = _native.DeviceBuffer(w.data_ptr(), w.numel(), True, w)
+        tmp_t = torch.empty(300_001, dtype=torch.uint8, device=dev)
+        tmp = _native.DeviceBuffer(tmp_t.data_ptr(), tmp_t.numel(), True, tmp_t)
+        assert buf.memmove(0, lead, tmp, 300_001) == 0
+        assert np.array_equal(w.cpu().numpy()[:300_001], want)
+
+
+def test_realign_batch_many_jobs(dev):
+    rng = np.random.default_rng(5)
+    src_host = rand_bytes(3_000_000, 2)
+    src = torch.from_numpy(src_host).to(dev)
+    jobs, spans, at = [], [], 0
+    dst = torch.full((4_000_000,), 0xA5, dtype=torch.uint8, device=dev)
+    for i in range(131):  # more than FSTX_BATCH_MAX: split into launches
+        n = int(rng.choice([0, 1, 4, 7, 16, 100, 4096, 20000, 70001]))
+        so = int(rng.integers(0, src_host.size - n))
+        at += int(rng.integers(0, 40))
+        jobs.append((dst.data_ptr() + at, src.data_ptr() + so, n))
+        spans.append((at, so, n))
+        at += n
+    _native.realign_copy_batch(jobs, stream())
+    got = dst.cpu().numpy()
+    want = np.full(4_000_000, 0xA5, dtype=np.uint8)
+    for at, so, n in spans:
+        want[at : at + n] = src_host[so : so + n]
+    assert np.array_equal(got, want)
+
+
+def test_realign_rejects_bad_arguments(dev):
+    a = torch.zeros(1024, dtype=torch.uint8, device=dev)
+    with pytest.raises(_native.NativeError):
+        _native.realign_copy(a.data_ptr() + 8, a.data_ptr(), 100)  # overlapping ranges
+    descs = (_native.FstxCopyDesc * 49)()
+    assert _native.lib().fstx_realign_copy_batch(descs, 49, None) == -10008  # FSTX_E_TOO_MANY
+
+
+def test_realign_full_size_c2_section(dev):
+    """Config C2's whole data section (709,646,336 bytes) shifted by 2 and by 10 bytes:
+    checked by 64-bit word sums and sampled windows instead of a full host copy."""
+    n = 709_646_336
+    g = torch.Generator(device=dev).manual_seed(42)
+    base = torch.randint(0, 256, (n + 4096,), dtype=torch.uint8, device=dev, generator=g)
+    out = torch.empty(n, dtype=torch.uint8, device=dev)
+    for m in (2, 10):
+        out.zero_()
+        _native.realign_copy(out.data_ptr(), base.data_ptr() + m, n, stream())
+        want = base[m : m + n]
+        assert torch.equal(out, want)
+
+
+# ---- slice extract ----------------------------------------------------------------------------
+
+
+def oracle_shard(raw: np.ndarray, dtype: str, shape, dim, rank, world):
+    return orc.shard_bytes(raw, dtype, list(shape), dim, rank, world)
+
+
+def gpu_shard(dev, raw: np.ndarray, itembits: int, shape, dim, rank, world, src_shift: int = 0):
+    """Cut rank's block with fstx_slice_copy; returns the shard bytes as numpy."""
+    block = -(-shape[dim] // world)
+    lo, hi = min(rank * block, shape[dim]), min((rank + 1) * block, shape[dim])
+    inner = int(np.prod(shape[dim + 1 :], dtype=np.int64)) * itembits // 8
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    seg, pitch, first = (hi - lo) * inner, shape[dim] * inner, lo * inner
+    host = np.full(raw.size + 64 + src_shift, 0x5A, dtype=np.uint8)
+    host[src_shift : src_shift + raw.size] = raw
+    src = torch.from_numpy(host).to(dev)
+    dst = torch.full((outer * seg + 128,), 0xA5, dtype=torch.uint8, device=dev)
+    _native.slice_copy(dst.data_ptr() + 64, src.data_ptr() + src_shift + first, outer, seg, pitch, stream())
+    got = dst.cpu().numpy()
+    assert (got[:64] == 0xA5).all() and (got[64 + outer * seg :] == 0xA5).all()
+    return got[64 : 64 + outer * seg]
+
+
+SHAPES = [
+    ((64, 64), "BF16"), ((5, 3), "BF16"), ((7, 250), "BF16"), ((33, 1000), "F16"), ((3, 4, 5), "F32"),
+    ((2, 3, 7), "U8"), ((128, 24), "F8_E4M3"), ((1, 9), "I64"), ((6,), "F32"), ((16, 8), "F16"),
+    ((40, 1280), "BF16"), ((9, 6, 10), "BF16"),
+]
+
+
+@pytest.mark.parametrize("shape,dtype", SHAPES)
+def test_slice_matches_oracle(dev, shape, dtype):
+    bits = orc.DTYPE_BITS[dtype]
+    raw = rand_bytes(int(np.prod(shape)) * bits // 8, hash(shape) % 1000)
+    for dim in range(len(shape)):
+        for world in (1, 2, 3, 4, 8):
+            for rank in range(world):
+                want, _ = oracle_shard(raw, dtype, shape, dim, rank, world)
+                for shift in (0, 16) if world != 4 else (0, 1, 2, 4, 8):
+                    got = gpu_shard(dev, raw, bits, shape, dim, rank, world, shift)
+                    assert np.array_equal(got, want), (shape, dtype, dim, world, rank, shift)
+
+
+def test_slice_batch_and_round_trip_full_size_c4(dev):
+    """Config C4 shapes at full size (Llama-2-13B, TP=4): the four ranks' shards,
+    cut in turn, concatenate back to the tensor (round trip), for dim 0 and dim 1."""
+    for shape, dim in [((5120, 5120), 0), ((5120, 5120), 1), ((13824, 5120), 0), ((5120, 13824), 1), ((32000, 5120), 0)]:
+        g = torch.Generator(device=dev).manual_seed(shape[0] + dim)
+        t = torch.randint(-32768, 32767, shape, dtype=torch.int16, device=dev, generator=g).view(torch.bfloat16)
+        world = 4
+        block = -(-shape[dim] // world)
+        inner = int(np.prod(shape[dim + 1 :], dtype=np.int64)) * 2
+        outer = int(np.prod(shape[:dim], dtype=np.int64))
+        parts, jobs = [], []
+        for rank in range(world):
+            out_shape = list(shape)
+            out_shape[dim] = block
+            p = torch.empty(out_shape, dtype=torch.bfloat16, device=dev)
+            parts.append(p)
+            jobs.append((p.data_ptr(), t.data_ptr() + rank * block * inner, outer, block * inner, shape[dim] * inner))
+        _native.slice_copy_batch(jobs, stream())
+        assert torch.equal(torch.cat(parts, dim=dim).view(torch.int16), t.view(torch.int16))
+        for rank in range(world):  # and each shard equals torch's own slice
+            sl = (slice(None),) * dim + (slice(rank * block, (rank + 1) * block),)
+            assert torch.equal(parts[rank].view(torch.int16), t[sl].contiguous().view(torch.int16))
+
+
+def test_slice_zero_sized_and_errors(dev):
+    a = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
+    _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 4, 0, 32, stream())
+    with pytest.raises(_native.NativeError):
+        _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 4, 64, 32, stream())  # pitch < segment
+    torch.cuda.synchronize()
