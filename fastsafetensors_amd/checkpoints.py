@@ -103,25 +103,25 @@ def _chunks(spec: TensorSpec) -> Iterable[Tuple[int, ...]]:
 
 
 def tensor_chunks(spec: TensorSpec, seed: int, device: str = "cpu") -> Iterable[torch.Tensor]:
-    """The tensor's values, chunk by chunk along dim 0, always as CPU tensors."""
+    """The tensor's values, chunk by chunk along dim 0, on ``device``."""
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)
     tdt = TORCH_DTYPE[spec.dtype]
     for i, shape in enumerate(_chunks(spec)):
         if spec.fill == "ones":
-            t = torch.ones(shape, dtype=tdt)
+            t = torch.ones(shape, dtype=tdt, device=device)
         elif spec.fill == "scale":
-            t = torch.full(shape, spec.scale, dtype=tdt)
+            t = torch.full(shape, spec.scale, dtype=tdt, device=device)
         elif spec.fill == "arange":
             n = 1
             for s in shape:
                 n *= s
-            t = (torch.arange(n, dtype=torch.int64) % 251).reshape(shape).to(tdt)
+            t = (torch.arange(n, dtype=torch.int64, device=device) % 251).reshape(shape).to(tdt)
         else:
             x = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * 0.02
             if spec.fill == "fp8":
                 x = (x / spec.scale).clamp_(-448.0, 448.0)
-            t = x.to(tdt).cpu()
+            t = x.to(tdt)
         yield t
 
 
@@ -135,15 +135,19 @@ def write_checkpoint(
     device: str = "cpu",
     reorder: bool = True,
     trailing: int = 0,
+    sha256: bool = True,
+    on_chunk: Optional[Callable[[TensorSpec, torch.Tensor], None]] = None,
 ) -> Dict[str, object]:
     """Write one file; returns ``{"path", "size", "header_length", "sha256", "specs"}``.
 
-    ``sha256`` covers the whole file.  ``trailing`` appends that many zero bytes
-    after the last tensor (the format allows it).
+    ``sha256`` covers the whole file (``None`` when switched off).  ``trailing``
+    appends that many zero bytes after the last tensor (the format allows it).
+    ``on_chunk(spec, chunk)`` sees every generated chunk on the generating
+    device before it is written, e.g. to keep checksums.
     """
     ordered = stock_order(specs) if reorder else list(specs)
     header = build_header(ordered, metadata, pad_mod, pad_rem)
-    digest = hashlib.sha256()
+    digest = hashlib.sha256() if sha256 else _NoDigest()
     tmp = f"{path}.{os.getpid()}.tmp"
     with open(tmp, "wb", buffering=0) as f:
         f.write(header)
@@ -152,7 +156,9 @@ def write_checkpoint(
             for t in tensor_chunks(spec, seed_base + i, device):
                 if not t.numel():
                     continue
-                raw = memoryview(t.contiguous().reshape(-1).view(torch.uint8).numpy())
+                if on_chunk is not None:
+                    on_chunk(spec, t)
+                raw = memoryview(t.contiguous().reshape(-1).view(torch.uint8).cpu().numpy())
                 f.write(raw)
                 digest.update(raw)
         if trailing:
@@ -162,6 +168,14 @@ def write_checkpoint(
     os.replace(tmp, path)
     return {"path": path, "size": size, "header_length": len(header), "sha256": digest.hexdigest(),
             "specs": ordered}
+
+
+class _NoDigest:
+    def update(self, _b) -> None:
+        pass
+
+    def hexdigest(self) -> None:
+        return None
 
 
 # ---- the benchmark shapes ---------------------------------------------------------
@@ -250,7 +264,8 @@ def configs(scale: float = 1.0) -> Dict[str, CheckpointConfig]:
 
 
 def write_config(
-    cfg: CheckpointConfig, directory: str, seed_base: int = 1234, device: str = "cpu"
+    cfg: CheckpointConfig, directory: str, seed_base: int = 1234, device: str = "cpu",
+    sha256: bool = True, on_chunk: Optional[Callable[[TensorSpec, torch.Tensor], None]] = None,
 ) -> List[Dict[str, object]]:
     """Write all files of ``cfg`` into ``directory``; returns ``write_checkpoint`` records."""
     os.makedirs(directory, exist_ok=True)
@@ -262,6 +277,7 @@ def write_config(
             write_checkpoint(
                 os.path.join(directory, name), specs, seed_base + 100_000 * k,
                 metadata={"format": "pt"}, pad_mod=8, pad_rem=cfg.pad_rem, device=device,
+                sha256=sha256, on_chunk=on_chunk,
             )
         )
     return out
