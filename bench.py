@@ -232,9 +232,11 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     stream = torch.cuda.current_stream().cuda_stream
     out: Dict[str, dict] = {}
 
-    def timed(launch, reps: int) -> List[float]:
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-        for a, b in evs:
+    def timed(launches) -> List[float]:
+        """Per-launch milliseconds: an event pair around each launch, all enqueued
+        back to back on the launch stream so that no launch waits for the host."""
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches]
+        for (a, b), launch in zip(evs, launches):
             a.record()
             launch()
             b.record()
@@ -269,9 +271,8 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
             _native.slice_copy_batch(part, stream)
     times, nbytes = [], []
     for _ in range(max(1, steps)):
-        for part, b in launches:
-            times += timed(lambda p=part: _native.slice_copy_batch(p, stream), 1)
-            nbytes.append(b)
+        times += timed([lambda p=part: _native.slice_copy_batch(p, stream) for part, _b in launches])
+        nbytes += [b for _p, b in launches]
     # parity at full size: the four ranks' blocks put side by side give the tensor back
     per_rank = len(specs)
     for i, s in enumerate(specs):
@@ -292,13 +293,23 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
 
     # -- realign: config C2's data section shifted by header_length % 16 = 10 bytes
     n = 709_646_336
-    window = torch.randint(0, 255, (n + 4096,), dtype=torch.uint8, device=dev)
-    dst = torch.empty(n, dtype=torch.uint8, device=dev)
+    cal = 1 << 30
+    window = torch.randint(0, 255, (cal + 4096,), dtype=torch.uint8, device=dev)
+    dst = torch.empty(cal, dtype=torch.uint8, device=dev)
     for _ in range(max(1, warmup)):
         _native.realign_copy(dst.data_ptr(), window.data_ptr() + 10, n, stream)
-    times = timed(lambda: _native.realign_copy(dst.data_ptr(), window.data_ptr() + 10, n, stream), max(3, steps))
-    if not torch.equal(dst, window[10 : 10 + n]):
+    times = timed([lambda: _native.realign_copy(dst.data_ptr(), window.data_ptr() + 10, n, stream)] * max(3, steps))
+    if not torch.equal(dst[:n], window[10 : 10 + n]):
         raise SystemExit("bench: realign copy result differs from the source bytes")
+    # plain copy of known size (source already aligned): the yardstick that the
+    # FETCH_SIZE / WRITE_SIZE counters of the other launches are scaled by
+    _native.realign_copy(dst.data_ptr(), window.data_ptr(), cal, stream)
+    cal_times = timed([lambda: _native.realign_copy(dst.data_ptr(), window.data_ptr(), cal, stream)] * 3)
+    out["calibration_copy"] = {
+        "workload": f"aligned copy of {cal} bytes (realign_kernel, shift 0, grid {cal // 16} lanes)",
+        "launches_timed": len(cal_times), "avg_launch_ms": sum(cal_times) / len(cal_times),
+        "bytes_per_launch": 2 * cal, "achieved_GBps": 2 * cal / 1e6 / (sum(cal_times) / len(cal_times)),
+    }
     avg_ms = sum(times) / len(times)
     out["realign_copy"] = {
         "workload": "C2 GPT-2-medium fp16 data section, 709,646,336 bytes, source shifted by 10 bytes",
@@ -386,6 +397,8 @@ def main() -> None:
     ap.add_argument("--keep", action="store_true", help="keep the generated checkpoint")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-kernels", action="store_true")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="run only the HBM kernel section (short; the command the counter profiles use)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this load path drives ONE GPU; run it with --gpus 1 "
@@ -396,6 +409,9 @@ def main() -> None:
     from fastsafetensors_amd import checkpoints as ck
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    if args.kernels_only:
+        print(json.dumps({"kernels": bench_kernels(args.steps, args.warmup)}), flush=True)
+        return
     cfg = ck.configs(1.0)[args.config]
     data_dir = os.path.join(args.dir, args.config)
     sums: Dict[str, Tuple[int, int]] = {}
@@ -418,14 +434,18 @@ def main() -> None:
         # ceilings of this box
         drop_cache(files)
         cold_frac = resident_fraction(files)
-        nb, dt = parallel_read(files, direct=True, threads=4, limit=6 << 30)
-        disk_direct = nb / 1e9 / dt
+        # best of a small sweep, every point on cold pages (O_DIRECT leaves the cache cold)
+        disk_direct, disk_point = 0.0, None
+        for th, blk in [(2, 4 << 20), (4, 4 << 20), (8, 4 << 20), (4, 16 << 20), (16, 1 << 20)]:
+            nb, dt = parallel_read(files, direct=True, threads=th, limit=3 << 30, block=blk)
+            if nb / 1e9 / dt > disk_direct:
+                disk_direct, disk_point = nb / 1e9 / dt, f"{th} threads x {blk >> 20} MiB"
         h2d = measure_h2d_peak()
         warm_cache(files)
         warm_frac = resident_fraction(files)
         nb, dt = parallel_read(files, direct=False, threads=16, limit=8 << 30)
         pagecache = nb / 1e9 / dt
-        log(f"[bench] ceilings: O_DIRECT read {disk_direct:.2f} GB/s, pinned H2D {h2d:.2f} GB/s, page cache {pagecache:.1f} GB/s "
+        log(f"[bench] ceilings: O_DIRECT read {disk_direct:.2f} GB/s ({disk_point}), pinned H2D {h2d:.2f} GB/s, page cache {pagecache:.1f} GB/s "
             f"(resident after drop {cold_frac:.3f}, after warm-up {warm_frac:.3f})")
 
         def steps_of(kind: str, n: int, check: bool) -> List[Dict[str, float]]:
@@ -475,12 +495,12 @@ def main() -> None:
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": f"{args.config}: {cfg.title}, {len(files)} files, {data_bytes} data bytes, "
+        "config": {"workload": f"{args.config}: {cfg.title}, {data_bytes} data bytes, "
                                f"read_mode=auto, {args.threads} I/O threads, {args.block_kb} KiB blocks"},
         "cold": cold_s,
         "warm": warm_s,
         "seconds_to_load": {"cold": cold_s["seconds_to_load_median"], "warm": warm_s["seconds_to_load_median"]},
-        "pipeline": {"disk_o_direct_GBps": disk_direct, "h2d_pinned_GBps": h2d, "page_cache_read_GBps": pagecache,
+        "pipeline": {"disk_o_direct_GBps": disk_direct, "disk_o_direct_best_point": disk_point, "h2d_pinned_GBps": h2d, "page_cache_read_GBps": pagecache,
                      "resident_after_drop": cold_frac, "resident_after_warmup": warm_frac,
                      "parity": f"{cold[0].get('verified_tensors', 0)} tensors checksum-verified on the GPU after a cold and a warm load"},
     }
