@@ -57,6 +57,7 @@ class FstxMetrics(ctypes.Structure):
             "stage_ns",
             "slot_wait_ns",
             "direct_fallbacks",
+            "direct_depth",
         )
     ]
 

@@ -68,6 +68,7 @@ inline uint64_t now_ns() {
 
 std::atomic<int> g_debug{0};
 std::atomic<int64_t> g_bounce_bytes{0};
+std::atomic<uint32_t> g_depth_hint{4}; // O_DIRECT depth the last adaptive context settled on
 
 // ---- NUMA ------------------------------------------------------------------
 
@@ -151,27 +152,66 @@ struct Slot {
     bool pending = false; // an async copy out of this slot may still be running
 };
 
-// counting semaphore bounding concurrent O_DIRECT preads
+// Bounds the O_DIRECT preads in flight.  Storage differs a lot in the queue depth
+// it wants (a virtio disk peaks at 2, an NVMe array at 32 or more), so unless
+// the caller fixes the depth, it is steered while reading: every window of
+// completed blocks yields a rate; a step that raised the rate is repeated, a
+// step that lowered it is undone, and a tie drifts towards fewer readers.
 class Gate {
   public:
-    explicit Gate(uint32_t n) : free_(n) {}
+    Gate(uint32_t start, uint32_t hi, bool adaptive)
+        : limit_(std::max(1u, std::min(start, hi))), hi_(std::max(1u, hi)), adaptive_(adaptive) {}
     void enter() {
         std::unique_lock<std::mutex> lk(m_);
-        cv_.wait(lk, [&] { return free_ > 0; });
-        --free_;
+        cv_.wait(lk, [&] { return busy_ < limit_; });
+        ++busy_;
     }
-    void leave() {
+    void leave(uint64_t bytes) {
         {
             std::lock_guard<std::mutex> lk(m_);
-            ++free_;
+            --busy_;
+            if (adaptive_) steer(bytes);
         }
-        cv_.notify_one();
+        cv_.notify_all();
+    }
+    uint32_t limit() {
+        std::lock_guard<std::mutex> lk(m_);
+        return limit_;
     }
 
   private:
+    void steer(uint64_t bytes) {
+        const uint64_t now = now_ns();
+        if (win_blocks_ == 0 || now - last_done_ > 50'000'000ull) { // first block, or reading paused
+            win_t0_ = now;
+            win_bytes_ = 0;
+            win_blocks_ = 0;
+            if (now - last_done_ > 50'000'000ull) last_rate_ = 0;
+        }
+        last_done_ = now;
+        win_bytes_ += bytes;
+        if (++win_blocks_ < std::max(16u, 6 * limit_) || now == win_t0_) return;
+        const double rate = (double)win_bytes_ / (double)(now - win_t0_);
+        if (last_rate_ > 0) {
+            if (rate < 0.98 * last_rate_) dir_ = -dir_;          // that step hurt: go back
+            else if (rate < 1.02 * last_rate_) dir_ = -1;        // no gain: prefer fewer readers
+        }
+        last_rate_ = rate;
+        int64_t next = (int64_t)limit_ + dir_;
+        if (next < 1) { next = 1; dir_ = 1; }
+        if (next > (int64_t)hi_) { next = hi_; dir_ = -1; }
+        limit_ = (uint32_t)next;
+        win_blocks_ = 0;
+    }
+
     std::mutex m_;
     std::condition_variable cv_;
-    uint32_t free_;
+    uint32_t limit_, hi_, busy_ = 0;
+    bool adaptive_;
+    int dir_ = 1;
+    double last_rate_ = 0;
+    uint64_t win_t0_ = 0, win_bytes_ = 0, last_done_ = 0;
+    uint32_t win_blocks_ = 0;
 };
 
 struct Counters {
@@ -205,6 +245,7 @@ struct fstx_ctx {
     int64_t next_request = 1;
 
     Counters ctr;
+    bool adaptive_depth = false;
     std::atomic<int64_t> fault_after{-1}; // test hook: fail the n-th block read with EIO
 };
 
@@ -283,7 +324,7 @@ struct Worker {
             uint64_t t0 = now_ns();
             int64_t got = pread_full(f.fd_direct, stage, want, window);
             uint64_t t1 = now_ns();
-            ctx->direct_gate->leave();
+            ctx->direct_gate->leave(got > 0 ? (uint64_t)got : 0);
             if (got == -EINVAL || got == -EFAULT || got == -EOPNOTSUPP) {
                 // this file cannot do O_DIRECT after all; stay buffered from here on
                 f.direct_ok.store(false, std::memory_order_relaxed);
@@ -452,7 +493,8 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (cfg.n_streams == 0) cfg.n_streams = 4;
     if (cfg.block_bytes == 0) cfg.block_bytes = kDefaultBlock;
     if (cfg.slots_per_thread == 0) cfg.slots_per_thread = 2;
-    if (cfg.max_direct_reads == 0) cfg.max_direct_reads = 4;
+    const bool adaptive_depth = cfg.max_direct_reads == 0;
+    if (adaptive_depth) cfg.max_direct_reads = g_depth_hint.load();
     if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 ||
         cfg.slots_per_thread > 64)
         return -FSTX_E_INVAL;
@@ -466,7 +508,8 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 
     std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
     ctx->cfg = cfg;
-    ctx->direct_gate.reset(new Gate(cfg.max_direct_reads));
+    ctx->adaptive_depth = adaptive_depth;
+    ctx->direct_gate.reset(new Gate(cfg.max_direct_reads, std::min(cfg.n_threads, 32u), adaptive_depth));
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
 
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
@@ -535,6 +578,7 @@ int fstx_ctx_destroy(fstx_ctx *ctx) {
     }
     ctx->q_cv.notify_all();
     for (std::thread &t : ctx->workers) t.join(); // workers drain the queue first
+    if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->limit());
     fstx_dev::set_device(ctx->cfg.device_id);
     for (auto s : ctx->streams) fstx_dev::stream_sync(s);
     for (auto &per : ctx->slots)
@@ -679,6 +723,7 @@ int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
     out->stage_ns = c.stage_ns.load();
     out->slot_wait_ns = c.slot_wait_ns.load();
     out->direct_fallbacks = c.direct_fallbacks.load();
+    out->direct_depth = ctx->direct_gate->limit();
     return 0;
 }
 

@@ -64,7 +64,8 @@ typedef struct fstx_config {
     uint32_t n_streams;      /* HIP copy streams shared by the workers (0 = default 4)           */
     uint64_t block_bytes;    /* bytes per read block = per ring slot, multiple of 4096 (0 = 4 MiB)*/
     uint32_t slots_per_thread; /* ring slots each worker cycles through (0 = default 2)          */
-    uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 4)      */
+    uint32_t max_direct_reads; /* O_DIRECT preads in flight at once; 0 = start at 4 and adapt to
+                                  the storage while reading, > 0 = fixed at this depth            */
 } fstx_config;
 
 typedef struct fstx_metrics {
@@ -77,6 +78,7 @@ typedef struct fstx_metrics {
     uint64_t stage_ns;            /* summed over workers: staging memcpy after O_DIRECT          */
     uint64_t slot_wait_ns;        /* summed over workers: waiting for a ring slot's last copy    */
     uint64_t direct_fallbacks;    /* blocks that asked for O_DIRECT but were read buffered       */
+    uint64_t direct_depth;        /* O_DIRECT preads currently allowed in flight                 */
 } fstx_metrics;
 
 /* ---- library-wide helpers ------------------------------------------------ */

@@ -1,0 +1,90 @@
+// SPDX-License-Identifier: Apache-2.0
+//
+// TEST INFRASTRUCTURE.  Drives the copy pipeline (built against the in-memory
+// device stand-in) from several caller threads at once; meant to be built with
+// -fsanitize=thread or -fsanitize=address.  Exit status 0 = every byte matched.
+//
+//   hostsim_driver <file> [rounds]
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <thread>
+#include <vector>
+
+#include <fcntl.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include "fstx.h"
+
+extern "C" void fstx_sim_set_copy_delay_us(int us);
+
+int main(int argc, char **argv) {
+    if (argc < 2) return 2;
+    const char *path = argv[1];
+    int rounds = argc > 2 ? std::atoi(argv[2]) : 3;
+    struct stat st;
+    if (stat(path, &st) != 0) return 2;
+    const uint64_t size = (uint64_t)st.st_size;
+    std::vector<char> truth(size);
+    {
+        int fd = open(path, O_RDONLY);
+        uint64_t got = 0;
+        while (got < size) {
+            ssize_t c = pread(fd, truth.data() + got, size - got, (off_t)got);
+            if (c <= 0) return 2;
+            got += (uint64_t)c;
+        }
+        close(fd);
+    }
+    fstx_sim_set_copy_delay_us(20);
+    std::atomic<int> bad{0};
+    for (int round = 0; round < rounds; ++round) {
+        fstx_config cfg{};
+        cfg.struct_size = sizeof cfg;
+        cfg.device_id = 0;
+        cfg.numa_node = -1;
+        cfg.n_threads = 2 + round * 3;
+        cfg.n_streams = 1 + round;
+        cfg.block_bytes = 4096u << (round * 2);
+        cfg.slots_per_thread = 1 + round % 2;
+        fstx_ctx *ctx = nullptr;
+        if (fstx_ctx_create(&cfg, &ctx) != 0) return 3;
+        std::vector<std::thread> callers;
+        for (int c = 0; c < 3; ++c) {
+            callers.emplace_back([&, c] {
+                std::mt19937_64 rng(round * 100 + c);
+                int64_t file = fstx_file_open(ctx, path, c % 3);
+                if (file < 0) { bad++; return; }
+                std::vector<char> dev(size + 64, 0x5a);
+                std::vector<int64_t> reqs;
+                std::vector<std::pair<uint64_t, uint64_t>> spans;
+                uint64_t at = 0;
+                while (at < size) {
+                    uint64_t len = 1 + rng() % (size / 5 + 1);
+                    if (at + len > size) len = size - at;
+                    int64_t r = fstx_submit_read(ctx, file, at, len, dev.data(), dev.size(), at + 7);
+                    if (r < 0) { bad++; break; }
+                    reqs.push_back(r);
+                    spans.push_back({at, len});
+                    at += len;
+                }
+                for (size_t i = 0; i < reqs.size(); ++i)
+                    if (fstx_wait_read(ctx, reqs[i]) != (int64_t)spans[i].second) bad++;
+                if (std::memcmp(dev.data() + 7, truth.data(), size) != 0) bad++;
+                if (fstx_file_close(ctx, file) != 0) bad++;
+            });
+        }
+        for (auto &t : callers) t.join();
+        fstx_metrics m;
+        fstx_get_metrics(ctx, &m);
+        if (m.bytes_copied != 3 * size) bad++;
+        if (fstx_ctx_destroy(ctx) != 0) bad++;
+    }
+    if (fstx_bounce_buffer_bytes() != 0) bad++;
+    std::printf("hostsim_driver: %s\n", bad.load() ? "MISMATCH" : "ok");
+    return bad.load() ? 1 : 0;
+}

@@ -1,0 +1,81 @@
+# SPDX-License-Identifier: Apache-2.0
+"""The shipped library loads and exports exactly what include/fstx.h declares.
+No GPU work is started here: only argument checks and host-side helpers."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+from fastsafetensors_amd import _native
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "fstx.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fstx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_the_same_functions():
+    assert declared_functions() == sorted(_native.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(_native.library_path()), "libfstx.so is not built"
+    raw = ctypes.CDLL(_native.library_path())
+    for name in declared_functions():
+        assert hasattr(raw, name), name
+    assert _native.lib().fstx_abi_version() == 1
+
+
+def test_constants_match_the_header():
+    text = open(os.path.join(ROOT, "include", "fstx.h")).read()
+    assert int(re.search(r"#define FSTX_BATCH_MAX (\d+)", text).group(1)) == _native.FSTX_BATCH_MAX
+    assert int(re.search(r"#define FSTX_ABI_VERSION (\d+)", text).group(1)) == _native.FSTX_ABI_VERSION
+    assert ctypes.sizeof(_native.FstxConfig) == 40 and ctypes.sizeof(_native.FstxMetrics) == 80
+    assert ctypes.sizeof(_native.FstxCopyDesc) == 24 and ctypes.sizeof(_native.FstxSliceDesc) == 40
+
+
+def test_host_helpers():
+    assert _native.get_alignment_size() == 4096  # reference: tests/smoke_import_cpp.py:34-40
+    assert _native.get_cpp_metrics().bounce_buffer_bytes == 0
+    p = _native.cpu_malloc(10_000)
+    assert p and p % 4096 == 0
+    ctypes.memset(p, 0x41, 16)
+    assert _native.read_buffer(p, 4) == b"AAAA"
+    _native.cpu_free(p)
+    assert _native.strerror(-10004).startswith("fstx: file ended")
+    assert "No such file" in _native.strerror(-2)
+    assert _native.strerror(0) == "ok"
+    assert _native.set_numa_node(-1) == 0
+    _native.set_debug_log(False)
+
+
+def test_argument_checks_need_no_gpu():
+    lib = _native.lib()
+    assert lib.fstx_realign_copy_batch(None, 0, None) == 0  # empty batch: nothing launched
+    assert lib.fstx_slice_copy_batch(None, 0, None) == 0
+    assert lib.fstx_realign_copy_batch(None, 3, None) == -10001
+    too_many = (_native.FstxCopyDesc * (_native.FSTX_BATCH_MAX + 1))()
+    assert lib.fstx_realign_copy_batch(too_many, len(too_many), None) == -10008
+    assert lib.fstx_ctx_create(None, None) == -10001
+    assert lib.fstx_ctx_destroy(None) == -10001
+    assert lib.fstx_get_device_pci_bus(0, None, 0) == -10001
+
+
+def test_without_a_gpu_the_product_refuses_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from fastsafetensors_amd import SafeTensorsFileLoader, SingleGroup
+
+    assert _native.device_count() == 0 and not _native.is_hip_found()
+    assert _native.get_device_pci_bus(0) == ""
+    with pytest.raises(Exception, match="HIP device"):
+        SafeTensorsFileLoader(SingleGroup(), "cpu")  # no CPU path behind the loader
+    with pytest.raises(Exception, match="no HIP device is visible"):
+        SafeTensorsFileLoader(SingleGroup(), "cuda:0")  # and no silent fallback either
+    with pytest.raises(_native.NativeError, match="no HIP device"):
+        _native.Reader(0)

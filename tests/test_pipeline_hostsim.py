@@ -1,0 +1,200 @@
+# SPDX-License-Identifier: Apache-2.0
+"""Host-side logic of the copy pipeline, without a GPU.
+
+``tests/hostsim`` links ``fstx_pipeline.cpp`` -- the very source that ships in
+libfstx.so -- against an in-memory stand-in for the GPU runtime whose streams
+run late and in order.  These tests drive that build through the C ABI: request
+splitting, ring reuse, every read mode, error paths, and the same under the
+thread and address sanitizers.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from fastsafetensors_amd import _native
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SIM_DIR = os.path.join(HERE, "hostsim")
+PIPELINE_SYMBOLS = [
+    n for n in _native.EXPORTED_SYMBOLS if not ("realign" in n or "slice" in n)
+]
+
+
+@pytest.fixture(scope="module")
+def sim():
+    if not os.path.exists(os.path.join(SIM_DIR, "libfstx_hostsim.so")):
+        subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
+    lib = ctypes.CDLL(os.path.join(SIM_DIR, "libfstx_hostsim.so"))
+    for name in PIPELINE_SYMBOLS:
+        restype, argtypes = _native._SIGNATURES[name]
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = restype, argtypes
+    lib.fstx_sim_set_copy_delay_us.argtypes = [ctypes.c_int]
+    lib.fstx_sim_fail_copy_after.argtypes = [ctypes.c_int64]
+    lib.fstx_sim_pinned_live.restype = ctypes.c_int64
+    lib.fstx_sim_set_copy_delay_us(30)
+    return lib
+
+
+@pytest.fixture(scope="module")
+def blob(tmp_path_factory):
+    path = str(tmp_path_factory.mktemp("sim") / "blob.bin")
+    data = np.random.default_rng(1).integers(0, 256, 9_000_011, dtype=np.uint8)
+    data.tofile(path)
+    return path, data
+
+
+def make_ctx(sim, **kw):
+    cfg = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, kw.get("threads", 4), kw.get("streams", 2),
+                             kw.get("block", 64 * 1024), kw.get("slots", 2), kw.get("depth", 0))
+    ctx = ctypes.c_void_p()
+    rc = sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(ctx))
+    assert rc == 0, rc
+    return ctx
+
+
+def metrics(sim, ctx):
+    m = _native.FstxMetrics()
+    assert sim.fstx_get_metrics(ctx, ctypes.byref(m)) == 0
+    return m
+
+
+@pytest.mark.parametrize("mode", [_native.READ_AUTO, _native.READ_BUFFERED, _native.READ_DIRECT])
+@pytest.mark.parametrize("block,threads,slots", [(4096, 3, 1), (64 * 1024, 4, 2), (1 << 20, 8, 2), (4 << 20, 2, 3)])
+def test_random_spans_land_byte_exact(sim, blob, mode, block, threads, slots):
+    path, data = blob
+    ctx = make_ctx(sim, block=block, threads=threads, slots=slots)
+    f = sim.fstx_file_open(ctx, path.encode(), mode)
+    assert f >= 1
+    rng = np.random.default_rng(block + threads)
+    dev = np.full(data.size + 100, 0xEE, dtype=np.uint8)
+    spans, at = [], 0
+    while at < data.size:
+        n = int(rng.integers(1, data.size // 7))
+        n = min(n, data.size - at)
+        spans.append((at, n, sim.fstx_submit_read(ctx, f, at, n, dev.ctypes.data, dev.size, at + 13)))
+        at += n
+    for _, n, req in spans:
+        assert req >= 1
+        assert sim.fstx_wait_read(ctx, req) == n
+    assert np.array_equal(dev[13 : 13 + data.size], data)
+    assert (dev[:13] == 0xEE).all() and (dev[13 + data.size :] == 0xEE).all()
+    m = metrics(sim, ctx)
+    assert m.bytes_read == data.size and m.bytes_copied == data.size
+    if mode == _native.READ_BUFFERED:
+        assert m.blocks_direct == 0
+    assert m.bounce_buffer_bytes == threads * slots * (block + 4096)
+    assert sim.fstx_bounce_buffer_bytes() == m.bounce_buffer_bytes
+    assert sim.fstx_file_close(ctx, f) == 0
+    assert sim.fstx_ctx_destroy(ctx) == 0
+    assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+
+
+def test_unaligned_window_start_and_zero_length(sim, blob):
+    path, data = blob
+    ctx = make_ctx(sim, block=8192)
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_DIRECT)
+    dev = np.zeros(50_000, dtype=np.uint8)
+    for off, n in [(1, 1), (4095, 2), (4097, 8191), (10, 40_000), (data.size - 5, 5), (0, 0)]:
+        dev[:] = 0
+        req = sim.fstx_submit_read(ctx, f, off, n, dev.ctypes.data, dev.size, 3)
+        assert sim.fstx_wait_read(ctx, req) == n
+        assert np.array_equal(dev[3 : 3 + n], data[off : off + n])
+        assert not dev[3 + n :].any()
+    sim.fstx_file_close(ctx, f)
+    sim.fstx_ctx_destroy(ctx)
+
+
+def test_error_paths(sim, blob, tmp_path):
+    path, data = blob
+    ctx = make_ctx(sim)
+    dev = np.zeros(1 << 20, dtype=np.uint8)
+    assert sim.fstx_file_open(ctx, b"/nonexistent/file", 0) == -2  # -ENOENT
+    assert "No such file" in sim.fstx_strerror(-2).decode()
+    f = sim.fstx_file_open(ctx, path.encode(), 0)
+    # destination range must fit the device buffer (std::out_of_range in the reference, ext.hpp:139-146)
+    assert sim.fstx_submit_read(ctx, f, 0, 2000, dev.ctypes.data, 1000, 0) == -_native_code("RANGE")
+    assert sim.fstx_submit_read(ctx, f, 0, 10, dev.ctypes.data, 1000, 995) == -_native_code("RANGE")
+    # reading past the end of the file fails at wait, never silently
+    req = sim.fstx_submit_read(ctx, f, data.size - 10, 20, dev.ctypes.data, dev.size, 0)
+    assert req >= 1 and sim.fstx_wait_read(ctx, req) == -_native_code("SHORT_READ")
+    assert sim.fstx_wait_read(ctx, req) == -_native_code("NO_REQ")  # ids are consumed
+    assert sim.fstx_submit_read(ctx, 999, 0, 10, dev.ctypes.data, dev.size, 0) == -_native_code("NO_REQ")
+    # file shrinks after open: the worker sees the short read
+    cut = str(tmp_path / "cut.bin")
+    data[:300_000].tofile(cut)
+    g = sim.fstx_file_open(ctx, cut.encode(), _native.READ_BUFFERED)
+    os.truncate(cut, 100_000)
+    req = sim.fstx_submit_read(ctx, g, 0, 300_000, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -_native_code("SHORT_READ")
+    # a close with a request outstanding is refused
+    req = sim.fstx_submit_read(ctx, f, 0, 100_000, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_file_close(ctx, f) == -16  # -EBUSY
+    assert sim.fstx_wait_read(ctx, req) == 100_000
+    assert sim.fstx_file_close(ctx, f) == 0 and sim.fstx_file_close(ctx, f) == -_native_code("NO_REQ")
+    # a failing device copy surfaces at wait
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+    sim.fstx_sim_fail_copy_after(3)
+    req = sim.fstx_submit_read(ctx, f, 0, 1 << 20, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -_native_code("HIP")
+    sim.fstx_sim_fail_copy_after(-1)
+    req = sim.fstx_submit_read(ctx, f, 0, 1 << 20, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == 1 << 20 and np.array_equal(dev, data[: 1 << 20])
+    assert sim.fstx_ctx_destroy(ctx) == 0  # also closes the file left open
+    assert sim.fstx_bounce_buffer_bytes() == 0
+    # bad configurations
+    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, 4, 2, 1000, 2, 0)  # block not a multiple of 4096
+    out = ctypes.c_void_p()
+    assert sim.fstx_ctx_create(ctypes.byref(bad), ctypes.byref(out)) == -_native_code("INVAL")
+    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 7, -1, 4, 2, 4096, 2, 0)  # no such device
+    assert sim.fstx_ctx_create(ctypes.byref(bad), ctypes.byref(out)) == -_native_code("INVAL")
+
+
+def _native_code(name: str) -> int:
+    return {"INVAL": 10001, "HIP": 10002, "RANGE": 10003, "SHORT_READ": 10004, "NO_REQ": 10005,
+            "CLOSED": 10006, "NO_DEVICE": 10007, "TOO_MANY": 10008}[name]
+
+
+def test_injected_read_fault(sim, blob):
+    path, data = blob
+    os.environ["FSTX_FAULT_READ_AFTER"] = "5"
+    try:
+        ctx = make_ctx(sim, block=64 * 1024)
+    finally:
+        del os.environ["FSTX_FAULT_READ_AFTER"]
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+    dev = np.zeros(data.size, dtype=np.uint8)
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -5  # -EIO from the sixth block
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == data.size and np.array_equal(dev, data)
+    sim.fstx_ctx_destroy(ctx)
+
+
+def test_destroy_with_requests_in_flight(sim, blob):
+    path, data = blob
+    sim.fstx_sim_set_copy_delay_us(300)
+    ctx = make_ctx(sim, block=4096, threads=2)
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+    dev = np.zeros(data.size, dtype=np.uint8)
+    for k in range(4):
+        assert sim.fstx_submit_read(ctx, f, k * 100_000, 100_000, dev.ctypes.data, dev.size, k * 100_000) >= 1
+    assert sim.fstx_ctx_destroy(ctx) == 0  # drains, never leaves a copy behind
+    sim.fstx_sim_set_copy_delay_us(30)
+    assert np.array_equal(dev[:400_000], data[:400_000])
+    assert sim.fstx_bounce_buffer_bytes() == 0
+
+
+@pytest.mark.parametrize("binary", ["hostsim_tsan.bin", "hostsim_asan.bin"])
+def test_pipeline_under_sanitizers(blob, binary):
+    exe = os.path.join(SIM_DIR, binary)
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
+    path, _ = blob
+    run = subprocess.run([exe, path, "3"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "Sanitizer" not in run.stderr, run.stderr
+    assert "hostsim_driver: ok" in run.stdout
