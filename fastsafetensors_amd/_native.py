@@ -20,6 +20,7 @@ _lib_lock = threading.Lock()
 FSTX_ABI_VERSION = 1
 FSTX_BATCH_MAX = 48
 READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
+ADAPTIVE_DEPTH = 1
 READ_MODES = {"auto": READ_AUTO, "buffered": READ_BUFFERED, "direct": READ_DIRECT}
 
 
@@ -41,6 +42,9 @@ class FstxConfig(ctypes.Structure):
         ("block_bytes", ctypes.c_uint64),
         ("slots_per_thread", ctypes.c_uint32),
         ("max_direct_reads", ctypes.c_uint32),
+        ("direct_read_bytes", ctypes.c_uint64),
+        ("flags", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
     ]
 
 
@@ -295,10 +299,12 @@ class Reader:
         block_bytes: int = 0,
         slots_per_thread: int = 0,
         max_direct_reads: int = 0,
+        direct_read_bytes: int = 0,
+        adaptive_depth: bool = False,
     ):
         cfg = FstxConfig(
             ctypes.sizeof(FstxConfig), device_id, numa_node, n_threads, n_streams, block_bytes,
-            slots_per_thread, max_direct_reads,
+            slots_per_thread, max_direct_reads, direct_read_bytes, ADAPTIVE_DEPTH if adaptive_depth else 0, 0,
         )
         handle = ctypes.c_void_p()
         _check("fstx_ctx_create", lib().fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(handle)))

@@ -215,6 +215,8 @@ def new_mi355x_file_copier(
     n_streams: int = 0,
     slots_per_thread: int = 0,
     max_direct_reads: int = 0,
+    direct_read_kb: Optional[int] = None,
+    adaptive_depth: bool = False,
     numa_node: Optional[int] = None,
     **kwargs,
 ) -> CopierConstructFunc:
@@ -241,6 +243,8 @@ def new_mi355x_file_copier(
         block_bytes=block_kb * 1024,
         slots_per_thread=slots_per_thread,
         max_direct_reads=max_direct_reads,
+        direct_read_bytes=(direct_read_kb or int(os.environ.get("FSTX_DIRECT_READ_KB", "0"))) * 1024,
+        adaptive_depth=adaptive_depth,
     )
 
     def construct(metadata: SafeTensorsMetadata, device: Device, framework: FrameworkOpBase) -> CopierInterface:

@@ -17,8 +17,9 @@
 //     moves on to its next slot, so the copy of block k overlaps the read of
 //     block k+1 (the event is waited only when the slot comes round again);
 //   * a block is read either from the page cache straight into the ring, or
-//     with O_DIRECT into an ordinary aligned staging block and then moved
-//     into the ring.  O_DIRECT cannot target the ring itself: device-visible
+//     with O_DIRECT -- one large pread covering a run of consecutive blocks,
+//     issued in ascending file order -- into an ordinary aligned staging block
+//     and then moved into the ring block by block.  O_DIRECT cannot target the ring itself: device-visible
 //     pinned memory is not backed by pages the block layer can pin, and
 //     the read fails with EFAULT.  In AUTO mode the choice is made per block
 //     from mincore() residency.
@@ -68,7 +69,7 @@ inline uint64_t now_ns() {
 
 std::atomic<int> g_debug{0};
 std::atomic<int64_t> g_bounce_bytes{0};
-std::atomic<uint32_t> g_depth_hint{4}; // O_DIRECT depth the last adaptive context settled on
+std::atomic<uint32_t> g_depth_hint{2}; // O_DIRECT depth the last adaptive context settled on
 
 // ---- NUMA ------------------------------------------------------------------
 
@@ -153,26 +154,26 @@ struct Slot {
 };
 
 // Bounds the O_DIRECT preads in flight.  Storage differs a lot in the queue depth
-// it wants (a virtio disk peaks at 2, an NVMe array at 32 or more), so unless
-// the caller fixes the depth, it is steered while reading: every window of
+// it wants (a virtio disk peaks at 2, an NVMe array at 32 or more); with
+// FSTX_ADAPTIVE_DEPTH the depth is steered while reading: every window of
 // completed blocks yields a rate; a step that raised the rate is repeated, a
-// step that lowered it is undone, and a tie drifts towards fewer readers.
+// step that lowered it is undone, and a change within the noise leaves the depth alone.
 class Gate {
   public:
     Gate(uint32_t start, uint32_t hi, bool adaptive)
         : limit_(std::max(1u, std::min(start, hi))), hi_(std::max(1u, hi)), adaptive_(adaptive) {}
-    void enter() {
-        std::unique_lock<std::mutex> lk(m_);
-        cv_.wait(lk, [&] { return busy_ < limit_; });
+    // take a token if one is free; callers that must start their reads in file
+    // order call this while they hold the block queue's lock
+    bool try_enter() {
+        std::lock_guard<std::mutex> lk(m_);
+        if (busy_ >= limit_) return false;
         ++busy_;
+        return true;
     }
     void leave(uint64_t bytes) {
-        {
-            std::lock_guard<std::mutex> lk(m_);
-            --busy_;
-            if (adaptive_) steer(bytes);
-        }
-        cv_.notify_all();
+        std::lock_guard<std::mutex> lk(m_);
+        --busy_;
+        if (adaptive_) steer(bytes);
     }
     uint32_t limit() {
         std::lock_guard<std::mutex> lk(m_);
@@ -192,12 +193,13 @@ class Gate {
         win_bytes_ += bytes;
         if (++win_blocks_ < std::max(16u, 6 * limit_) || now == win_t0_) return;
         const double rate = (double)win_bytes_ / (double)(now - win_t0_);
+        int step = dir_;
         if (last_rate_ > 0) {
-            if (rate < 0.98 * last_rate_) dir_ = -dir_;          // that step hurt: go back
-            else if (rate < 1.02 * last_rate_) dir_ = -1;        // no gain: prefer fewer readers
+            if (rate < 0.92 * last_rate_) step = dir_ = -dir_;   // that step hurt: go back
+            else if (rate < 1.08 * last_rate_) step = 0;         // within the noise: stay
         }
         last_rate_ = rate;
-        int64_t next = (int64_t)limit_ + dir_;
+        int64_t next = (int64_t)limit_ + step;
         if (next < 1) { next = 1; dir_ = 1; }
         if (next > (int64_t)hi_) { next = hi_; dir_ = -1; }
         limit_ = (uint32_t)next;
@@ -205,7 +207,6 @@ class Gate {
     }
 
     std::mutex m_;
-    std::condition_variable cv_;
     uint32_t limit_, hi_, busy_ = 0;
     bool adaptive_;
     int dir_ = 1;
@@ -245,6 +246,11 @@ struct fstx_ctx {
     int64_t next_request = 1;
 
     Counters ctr;
+    uint64_t direct_bytes = 0; // bytes one O_DIRECT pread may cover
+    // ordinary page-backed blocks that O_DIRECT reads land in; handed out together
+    // with the read token (under q_mutex), returned after the last byte left for the ring
+    std::vector<char *> stage_free;
+    uint32_t stage_made = 0, stage_max = 0;
     bool adaptive_depth = false;
     std::atomic<int64_t> fault_after{-1}; // test hook: fail the n-th block read with EIO
 };
@@ -290,122 +296,234 @@ bool block_is_cached(const FileEntry &f, uint64_t lo, uint64_t hi) {
 struct Worker {
     fstx_ctx *ctx;
     uint32_t index;
-    char *stage = nullptr; // ordinary page-backed memory for O_DIRECT reads
+    char *stage = nullptr; // staging block borrowed from the context for one O_DIRECT read
+    std::vector<Slot> *mine = nullptr;
+    size_t turn = 0;
+    uint32_t stream_ix = 0;
+    fstx_dev::stream_t stream = nullptr;
 
-    ~Worker() { std::free(stage); }
-
-    // Fill `slot` so that payload byte i sits at slot + (file_off - window) + i.
-    // Returns the in-slot offset of the payload or a negative status.
-    int64_t fill(const Block &b, Slot &slot) {
+    bool wants_direct(const Block &b) {
         FileEntry &f = *b.req->file;
-        const uint64_t window = align_down(b.file_off, kPage);
-        const uint64_t in_slot = b.file_off - window;
-
-        int64_t hook = ctx->fault_after.load(std::memory_order_relaxed);
-        if (hook >= 0 && ctx->fault_after.fetch_sub(1) == 0) return -EIO;
-
-        bool direct = false;
         if (f.fd_direct >= 0 && f.direct_ok.load(std::memory_order_relaxed)) {
-            if (f.mode == FSTX_READ_DIRECT) direct = true;
-            else if (f.mode == FSTX_READ_AUTO)
-                direct = !block_is_cached(f, b.file_off, b.file_off + b.len);
+            if (f.mode == FSTX_READ_DIRECT) return true;
+            if (f.mode == FSTX_READ_AUTO) return !block_is_cached(f, b.file_off, b.file_off + b.len);
         } else if (f.mode == FSTX_READ_DIRECT) {
             ctx->ctr.direct_fallbacks.fetch_add(1, std::memory_order_relaxed);
         }
+        return false;
+    }
 
-        if (direct) {
-            if (!stage && posix_memalign(reinterpret_cast<void **>(&stage), kPage,
-                                         ctx->cfg.block_bytes + kPage) != 0) {
-                stage = nullptr;
-                return -ENOMEM;
+    bool fault_hook() {
+        int64_t hook = ctx->fault_after.load(std::memory_order_relaxed);
+        return hook >= 0 && ctx->fault_after.fetch_sub(1) == 0;
+    }
+
+    // next ring slot of this worker, its previous copy finished
+    int64_t take_slot(Slot **out) {
+        Slot &slot = (*mine)[turn];
+        turn = (turn + 1) % mine->size();
+        int64_t status = 0;
+        if (slot.pending) {
+            if (fstx_dev::event_ready(slot.ev) != 1) {
+                uint64_t t0 = now_ns();
+                status = fstx_dev::event_sync(slot.ev);
+                ctx->ctr.slot_wait_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
             }
-            const uint64_t want = align_up(in_slot + b.len, kPage);
-            ctx->direct_gate->enter();
-            uint64_t t0 = now_ns();
-            int64_t got = pread_full(f.fd_direct, stage, want, window);
-            uint64_t t1 = now_ns();
-            ctx->direct_gate->leave(got > 0 ? (uint64_t)got : 0);
-            if (got == -EINVAL || got == -EFAULT || got == -EOPNOTSUPP) {
-                // this file cannot do O_DIRECT after all; stay buffered from here on
-                f.direct_ok.store(false, std::memory_order_relaxed);
-                ctx->ctr.direct_fallbacks.fetch_add(1, std::memory_order_relaxed);
-                direct = false;
-            } else {
-                if (got < 0) return got;
-                if ((uint64_t)got < in_slot + b.len) return -FSTX_E_SHORT_READ;
-                std::memcpy(slot.host + in_slot, stage + in_slot, b.len);
-                uint64_t t2 = now_ns();
-                ctx->ctr.read_ns.fetch_add(t1 - t0, std::memory_order_relaxed);
-                ctx->ctr.stage_ns.fetch_add(t2 - t1, std::memory_order_relaxed);
-                ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
-            }
+            slot.pending = false;
         }
-        if (!direct) {
-            uint64_t t0 = now_ns();
-            int64_t got = pread_full(f.fd_buffered, slot.host + in_slot, b.len, b.file_off);
-            ctx->ctr.read_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
-            if (got < 0) return got;
-            if ((uint64_t)got < b.len) return -FSTX_E_SHORT_READ;
-            ctx->ctr.blocks_buffered.fetch_add(1, std::memory_order_relaxed);
-        }
+        *out = &slot;
+        return status;
+    }
+
+    // enqueue slot -> device for block b; payload sits at slot.host + at
+    int64_t ship(const Block &b, Slot &slot, uint64_t at) {
+        int64_t status = fstx_dev::copy_to_device_async(b.dev, slot.host + at, b.len, stream);
+        if (status < 0) return status;
+        slot.pending = true;
+        status = fstx_dev::event_record(slot.ev, stream);
+        b.req->stream_mask.fetch_or(1ull << stream_ix, std::memory_order_relaxed);
+        ctx->ctr.bytes_copied.fetch_add(b.len, std::memory_order_relaxed);
         ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
-        return (int64_t)in_slot;
+        return status;
+    }
+
+    void finish(const Block &b, int64_t status) {
+        if (status < 0) {
+            int64_t none = 0;
+            b.req->error.compare_exchange_strong(none, status);
+        }
+        if (b.req->blocks_left.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+            std::lock_guard<std::mutex> lk(ctx->done_mutex);
+            ctx->done_cv.notify_all();
+        }
+    }
+
+    // page-cache read straight into a ring slot
+    int64_t do_buffered(const Block &b) {
+        if (fault_hook()) return -EIO;
+        Slot *slot = nullptr;
+        int64_t status = take_slot(&slot);
+        if (status < 0) return status;
+        const uint64_t at = b.file_off % kPage;
+        uint64_t t0 = now_ns();
+        int64_t got = pread_full(b.req->file->fd_buffered, slot->host + at, b.len, b.file_off);
+        ctx->ctr.read_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
+        if (got < 0) return got;
+        if ((uint64_t)got < b.len) return -FSTX_E_SHORT_READ;
+        ctx->ctr.blocks_buffered.fetch_add(1, std::memory_order_relaxed);
+        return ship(b, *slot, at);
+    }
+
+    // hand the O_DIRECT token back and wake a worker that waits for it
+    void release_token(uint64_t bytes) {
+        ctx->direct_gate->leave(bytes);
+        {
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        }
+        ctx->q_cv.notify_all();
+    }
+
+    // One O_DIRECT pread covers a run of consecutive blocks of one request (large
+    // requests amortise the per-request latency of the storage); the blocks then
+    // go through the ring one by one.  Returns false when the file turned out
+    // not to support O_DIRECT and the run has to be read buffered.
+    bool do_direct(std::vector<Block> &run, std::vector<int64_t> &status) {
+        FileEntry &f = *run.front().req->file;
+        const uint64_t window = align_down(run.front().file_off, kPage);
+        const uint64_t end = run.back().file_off + run.back().len;
+        const uint64_t want = align_up(end, kPage) - window;
+        if (!stage) {
+            release_token(0);
+            status.assign(run.size(), -ENOMEM);
+            return true;
+        }
+        if (fault_hook()) {
+            release_token(0);
+            return_stage();
+            status.assign(run.size(), -EIO);
+            return true;
+        }
+        uint64_t t0 = now_ns();
+        int64_t got = pread_full(f.fd_direct, stage, want, window);
+        uint64_t t1 = now_ns();
+        release_token(got > 0 ? (uint64_t)got : 0);
+        if (got == -EINVAL || got == -EFAULT || got == -EOPNOTSUPP) {
+            f.direct_ok.store(false, std::memory_order_relaxed);
+            ctx->ctr.direct_fallbacks.fetch_add(run.size(), std::memory_order_relaxed);
+            return_stage();
+            return false;
+        }
+        ctx->ctr.read_ns.fetch_add(t1 - t0, std::memory_order_relaxed);
+        for (size_t i = 0; i < run.size(); ++i) {
+            const Block &b = run[i];
+            if (got < 0) { status[i] = got; continue; }
+            if (window + (uint64_t)got < b.file_off + b.len) { status[i] = -FSTX_E_SHORT_READ; continue; }
+            Slot *slot = nullptr;
+            if ((status[i] = take_slot(&slot)) < 0) continue;
+            uint64_t t2 = now_ns();
+            std::memcpy(slot->host, stage + (b.file_off - window), b.len);
+            ctx->ctr.stage_ns.fetch_add(now_ns() - t2, std::memory_order_relaxed);
+            ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
+            status[i] = ship(b, *slot, 0);
+        }
+        return_stage();
+        return true;
+    }
+
+    // called with q_mutex held: borrow a staging block, making one if the pool may still grow
+    bool borrow_stage() {
+        if (!ctx->stage_free.empty()) {
+            stage = ctx->stage_free.back();
+            ctx->stage_free.pop_back();
+            return true;
+        }
+        if (ctx->stage_made >= ctx->stage_max) return false;
+        void *p = nullptr;
+        if (posix_memalign(&p, kPage, ctx->direct_bytes + 2 * kPage) != 0) p = nullptr;
+        stage = static_cast<char *>(p); // nullptr: the read reports ENOMEM
+        if (p) ++ctx->stage_made;
+        return true;
+    }
+
+    void return_stage() {
+        if (!stage) return;
+        {
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+            ctx->stage_free.push_back(stage);
+        }
+        stage = nullptr;
+        ctx->q_cv.notify_all();
     }
 
     void run() {
         bind_thread_to_node(ctx->cfg.numa_node);
-        int dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
-        std::vector<Slot> &mine = ctx->slots[index];
-        const uint32_t stream_ix = index % (uint32_t)ctx->streams.size();
-        fstx_dev::stream_t stream = ctx->streams[stream_ix];
-        size_t turn = 0;
+        const int64_t dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
+        mine = &ctx->slots[index];
+        stream_ix = index % (uint32_t)ctx->streams.size();
+        stream = ctx->streams[stream_ix];
+        std::vector<Block> run;
+        std::vector<int64_t> status;
         for (;;) {
-            Block b;
+            run.clear();
+            bool direct = false;
             {
+                // Blocks leave the queue in file order.  A block that needs O_DIRECT is
+                // taken together with its token, under this lock, so that the reads reach
+                // the storage in ascending order too (storage that detects sequential
+                // streams serves them about twice as fast as the same requests shuffled).
                 std::unique_lock<std::mutex> lk(ctx->q_mutex);
-                ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty(); });
-                if (ctx->queue.empty()) break; // closing and drained
-                b = std::move(ctx->queue.front());
+                for (;;) {
+                    ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty(); });
+                    if (ctx->queue.empty()) break; // closing and drained
+                    const Block &head = ctx->queue.front();
+                    direct = dev_rc == 0 && head.req->error.load(std::memory_order_relaxed) == 0 &&
+                             wants_direct(head);
+                    if (!direct) break;
+                    if ((!ctx->stage_free.empty() || ctx->stage_made < ctx->stage_max) &&
+                        ctx->direct_gate->try_enter()) {
+                        borrow_stage();
+                        break;
+                    }
+                    ctx->q_cv.wait(lk); // tokens or staging blocks are all out: wait for one to come back
+                }
+                if (ctx->queue.empty()) break;
+                run.push_back(std::move(ctx->queue.front()));
                 ctx->queue.pop_front();
+                if (direct) {
+                    // extend the run with the blocks that follow it in the file
+                    uint64_t bytes = run[0].len + run[0].file_off % kPage;
+                    while (!ctx->queue.empty()) {
+                        const Block &nx = ctx->queue.front();
+                        const Block &last = run.back();
+                        if (nx.req != last.req || nx.file_off != last.file_off + last.len ||
+                            bytes + nx.len > ctx->direct_bytes)
+                            break;
+                        bytes += nx.len;
+                        run.push_back(std::move(ctx->queue.front()));
+                        ctx->queue.pop_front();
+                    }
+                }
             }
-            int64_t status = dev_rc;
             // once a request has failed, its remaining blocks are only counted off
-            if (status == 0 && b.req->error.load(std::memory_order_relaxed) == 0) {
-                Slot &slot = mine[turn];
-                turn = (turn + 1) % mine.size();
-                if (slot.pending) {
-                    if (fstx_dev::event_ready(slot.ev) != 1) {
-                        uint64_t t0 = now_ns();
-                        status = fstx_dev::event_sync(slot.ev);
-                        ctx->ctr.slot_wait_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
-                    }
-                    slot.pending = false;
+            if (dev_rc < 0 || run[0].req->error.load(std::memory_order_relaxed) != 0) {
+                if (direct) {
+                    release_token(0);
+                    return_stage();
                 }
-                if (status == 0) {
-                    int64_t in_slot = fill(b, slot);
-                    if (in_slot < 0) status = in_slot;
-                    else {
-                        status = fstx_dev::copy_to_device_async(b.dev, slot.host + in_slot, b.len, stream);
-                        if (status == 0) {
-                            slot.pending = true;
-                            status = fstx_dev::event_record(slot.ev, stream);
-                            b.req->stream_mask.fetch_or(1ull << stream_ix, std::memory_order_relaxed);
-                            ctx->ctr.bytes_copied.fetch_add(b.len, std::memory_order_relaxed);
-                        }
-                    }
+                for (Block &b : run) finish(b, dev_rc);
+                continue;
+            }
+            if (direct) {
+                status.assign(run.size(), 0);
+                if (do_direct(run, status)) {
+                    for (size_t i = 0; i < run.size(); ++i) finish(run[i], status[i]);
+                    continue;
                 }
             }
-            if (status < 0) {
-                int64_t none = 0;
-                b.req->error.compare_exchange_strong(none, status);
-            }
-            if (b.req->blocks_left.fetch_sub(1, std::memory_order_acq_rel) == 1) {
-                std::lock_guard<std::mutex> lk(ctx->done_mutex);
-                ctx->done_cv.notify_all();
-            }
+            for (Block &b : run) finish(b, do_buffered(b));
         }
         // leave no copy in flight that still reads this worker's slots
-        for (Slot &s : mine)
+        for (Slot &s : *mine)
             if (s.pending) {
                 fstx_dev::event_sync(s.ev);
                 s.pending = false;
@@ -493,8 +611,10 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (cfg.n_streams == 0) cfg.n_streams = 4;
     if (cfg.block_bytes == 0) cfg.block_bytes = kDefaultBlock;
     if (cfg.slots_per_thread == 0) cfg.slots_per_thread = 2;
-    const bool adaptive_depth = cfg.max_direct_reads == 0;
-    if (adaptive_depth) cfg.max_direct_reads = g_depth_hint.load();
+    const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
+    if (cfg.max_direct_reads == 0) cfg.max_direct_reads = adaptive_depth ? g_depth_hint.load() : 1;
+    if (cfg.direct_read_bytes == 0) cfg.direct_read_bytes = 64ull << 20;
+    cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
     if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 ||
         cfg.slots_per_thread > 64)
         return -FSTX_E_INVAL;
@@ -509,6 +629,8 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
     ctx->cfg = cfg;
     ctx->adaptive_depth = adaptive_depth;
+    ctx->direct_bytes = cfg.direct_read_bytes;
+    ctx->stage_max = (adaptive_depth ? std::min(cfg.n_threads, 8u) : std::min(cfg.max_direct_reads, cfg.n_threads)) + 2;
     ctx->direct_gate.reset(new Gate(cfg.max_direct_reads, std::min(cfg.n_threads, 32u), adaptive_depth));
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
 
@@ -585,6 +707,7 @@ int fstx_ctx_destroy(fstx_ctx *ctx) {
         for (Slot &s : per) fstx_dev::event_destroy(s.ev);
     for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
     for (auto &kv : ctx->files) release_file(*kv.second);
+    for (char *p : ctx->stage_free) std::free(p);
     fstx_dev::host_free(ctx->ring);
     fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
     delete ctx;

@@ -150,7 +150,7 @@ class SafeTensorsFileLoader(BaseSafeTensorsFileLoader):
         nogds: accepted for compatibility; there is one copier.
         kwargs: forwarded to the copier factory (``read_mode``, ``layout``,
             ``block_size_kb``, ``n_streams``, ``slots_per_thread``,
-            ``max_direct_reads``, ``numa_node``).
+            ``max_direct_reads``, ``direct_read_kb``, ``adaptive_depth``, ``numa_node``).
 
     Example:
         >>> loader = SafeTensorsFileLoader(SingleGroup(), "cuda:0")

@@ -64,9 +64,15 @@ typedef struct fstx_config {
     uint32_t n_streams;      /* HIP copy streams shared by the workers (0 = default 4)           */
     uint64_t block_bytes;    /* bytes per read block = per ring slot, multiple of 4096 (0 = 4 MiB)*/
     uint32_t slots_per_thread; /* ring slots each worker cycles through (0 = default 2)          */
-    uint32_t max_direct_reads; /* O_DIRECT preads in flight at once; 0 = start at 4 and adapt to
-                                  the storage while reading, > 0 = fixed at this depth            */
+    uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 1)      */
+    uint64_t direct_read_bytes; /* bytes one O_DIRECT pread covers: a run of consecutive blocks,
+                                   multiple of block_bytes (0 = 64 MiB)                          */
+    uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH                                              */
+    uint32_t reserved;
 } fstx_config;
+
+/* fstx_config.flags: steer max_direct_reads while reading (start value = max_direct_reads) */
+#define FSTX_ADAPTIVE_DEPTH 1u
 
 typedef struct fstx_metrics {
     uint64_t bounce_buffer_bytes; /* pinned ring bytes currently allocated by this context       */

@@ -51,6 +51,8 @@ int main(int argc, char **argv) {
         cfg.n_streams = 1 + round;
         cfg.block_bytes = 4096u << (round * 2);
         cfg.slots_per_thread = 1 + round % 2;
+        cfg.direct_read_bytes = round == 1 ? 0 : cfg.block_bytes * 3;
+        cfg.flags = round == 2 ? FSTX_ADAPTIVE_DEPTH : 0;
         fstx_ctx *ctx = nullptr;
         if (fstx_ctx_create(&cfg, &ctx) != 0) return 3;
         std::vector<std::thread> callers;

@@ -33,7 +33,7 @@ def test_constants_match_the_header():
     text = open(os.path.join(ROOT, "include", "fstx.h")).read()
     assert int(re.search(r"#define FSTX_BATCH_MAX (\d+)", text).group(1)) == _native.FSTX_BATCH_MAX
     assert int(re.search(r"#define FSTX_ABI_VERSION (\d+)", text).group(1)) == _native.FSTX_ABI_VERSION
-    assert ctypes.sizeof(_native.FstxConfig) == 40 and ctypes.sizeof(_native.FstxMetrics) == 80
+    assert ctypes.sizeof(_native.FstxConfig) == 56 and ctypes.sizeof(_native.FstxMetrics) == 80
     assert ctypes.sizeof(_native.FstxCopyDesc) == 24 and ctypes.sizeof(_native.FstxSliceDesc) == 40
 
 

@@ -49,7 +49,8 @@ def blob(tmp_path_factory):
 
 def make_ctx(sim, **kw):
     cfg = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, kw.get("threads", 4), kw.get("streams", 2),
-                             kw.get("block", 64 * 1024), kw.get("slots", 2), kw.get("depth", 0))
+                             kw.get("block", 64 * 1024), kw.get("slots", 2), kw.get("depth", 0),
+                             kw.get("direct_bytes", 0), kw.get("flags", 0), 0)
     ctx = ctypes.c_void_p()
     rc = sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(ctx))
     assert rc == 0, rc
@@ -63,10 +64,11 @@ def metrics(sim, ctx):
 
 
 @pytest.mark.parametrize("mode", [_native.READ_AUTO, _native.READ_BUFFERED, _native.READ_DIRECT])
-@pytest.mark.parametrize("block,threads,slots", [(4096, 3, 1), (64 * 1024, 4, 2), (1 << 20, 8, 2), (4 << 20, 2, 3)])
-def test_random_spans_land_byte_exact(sim, blob, mode, block, threads, slots):
+@pytest.mark.parametrize("block,threads,slots,direct_bytes,flags", [
+    (4096, 3, 1, 4096, 0), (64 * 1024, 4, 2, 0, 1), (1 << 20, 8, 2, 3 << 20, 0), (4 << 20, 2, 3, 0, 0), (8192, 5, 1, 1 << 20, 1)])
+def test_random_spans_land_byte_exact(sim, blob, mode, block, threads, slots, direct_bytes, flags):
     path, data = blob
-    ctx = make_ctx(sim, block=block, threads=threads, slots=slots)
+    ctx = make_ctx(sim, block=block, threads=threads, slots=slots, direct_bytes=direct_bytes, flags=flags)
     f = sim.fstx_file_open(ctx, path.encode(), mode)
     assert f >= 1
     rng = np.random.default_rng(block + threads)
@@ -146,10 +148,10 @@ def test_error_paths(sim, blob, tmp_path):
     assert sim.fstx_ctx_destroy(ctx) == 0  # also closes the file left open
     assert sim.fstx_bounce_buffer_bytes() == 0
     # bad configurations
-    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, 4, 2, 1000, 2, 0)  # block not a multiple of 4096
+    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, 4, 2, 1000, 2, 0, 0, 0, 0)  # block not a multiple of 4096
     out = ctypes.c_void_p()
     assert sim.fstx_ctx_create(ctypes.byref(bad), ctypes.byref(out)) == -_native_code("INVAL")
-    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 7, -1, 4, 2, 4096, 2, 0)  # no such device
+    bad = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 7, -1, 4, 2, 4096, 2, 0, 0, 0, 0)  # no such device
     assert sim.fstx_ctx_create(ctypes.byref(bad), ctypes.byref(out)) == -_native_code("INVAL")
 
 
