@@ -120,7 +120,8 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 
 def library_path() -> str:
-    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+    """``libfstx.so`` next to this file, or the build named by ``FSTX_LIBRARY``."""
+    return os.environ.get("FSTX_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 
 
 def lib() -> ctypes.CDLL:

@@ -31,6 +31,8 @@ def command() -> List[str]:
     return [
         hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        # the kernels' leading scalar argument (granule_log2) arrives in a register
+        "-mllvm", "-amdgpu-kernarg-preload-count=1",
         f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
         "-o", OUTPUT, *[os.path.join(CSRC, s) for s in SOURCES], "-lpthread",
     ]
