@@ -224,6 +224,55 @@ def run_load(files: List[str], read_mode: str, threads: int, block_kb: int, veri
     return out
 
 
+# ---- tensor-parallel extraction through the loader API ---------------------------------------------------
+
+
+def bench_tp_extract(files: List[str], world: int, threads: int, block_kb: int) -> dict:
+    """``FilesBufferOnDevice.as_dict`` for every rank of a TP=``world`` group in turn
+    (a stub group reports rank r of ``world``): wall time from the call to the device
+    synchronize after it, inputs resident in HBM.  Checked by putting the ranks'
+    blocks side by side and comparing with the whole tensors."""
+    import torch
+    from collections import OrderedDict
+
+    from fastsafetensors_amd import SafeTensorsFileLoader, SingleGroup, StubProcessGroup
+    from fastsafetensors_amd import checkpoints as ck
+
+    whole_loader = SafeTensorsFileLoader(SingleGroup(), "cuda:0", max_threads=threads, block_size_kb=block_kb)
+    whole_loader.add_filenames({0: files})
+    whole = whole_loader.copy_files_to_device()
+    per_rank, secs, moved = [], [], 0
+    for rank in range(world):
+        loader = SafeTensorsFileLoader(StubProcessGroup(rank, world), "cuda:0", max_threads=threads,
+                                       block_size_kb=block_kb)
+        loader.add_filenames({rank: files})
+        bufs = loader.copy_files_to_device()
+        dims = OrderedDict((k, ck.llama_shard_dim(k)) for k in loader.get_keys())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = bufs.as_dict(dims)
+        torch.cuda.synchronize()
+        secs.append(time.perf_counter() - t0)
+        moved += sum(2 * t.get_raw().numel() * t.get_raw().element_size() for t in out.values())
+        per_rank.append({k: t.get_raw() for k, t in out.items()})
+        bufs.close()
+        loader.close()
+    checked = 0
+    for key, dim in dims.items():
+        full = whole.get_tensor(key)
+        got = per_rank[0][key] if dim < 0 else torch.cat([per_rank[r][key] for r in range(world)], dim=dim)
+        if got.shape != full.shape or not torch.equal(got.view(torch.uint8), full.view(torch.uint8)):
+            raise SystemExit(f"bench: TP blocks of {key} do not reassemble to the tensor")
+        checked += 1
+    whole.close()
+    whole_loader.close()
+    total = sum(secs)
+    return {"workload": f"as_dict of {len(dims)} tensors for each of {world} ranks (rows of q/k/v/gate/up/embed/lm_head, "
+                        f"columns of o/down, copies of the rest)",
+            "seconds_per_rank": secs, "algorithmic_bytes": moved, "GBps": moved / 1e9 / total,
+            "tensors_reassembled_and_compared": checked}
+
+
 # ---- kernels ------------------------------------------------------------------------------------------
 
 
@@ -503,6 +552,8 @@ def main() -> None:
         steps_of("warm", args.warmup, False)
         warm = steps_of("warm", args.steps, True)
 
+        tp = bench_tp_extract(files, 4, args.threads, args.block_kb)
+        log(f"[bench] TP=4 as_dict over the resident checkpoint: {tp['GBps']:.0f} GB/s, seconds per rank {[round(x, 4) for x in tp['seconds_per_rank']]}")
         kernels = {} if args.skip_kernels else bench_kernels(args.steps, args.warmup)
         base = None if args.skip_cpu_baseline else cpu_baseline(files)
     finally:
@@ -549,6 +600,7 @@ def main() -> None:
                      "resident_after_drop": cold_frac, "resident_after_warmup": warm_frac,
                      "parity": f"{cold[0].get('verified_tensors', 0)} tensors checksum-verified on the GPU after a cold and a warm load"},
     }
+    line["tp_extract"] = tp
     if kernels:
         k = kernels["slice_extract"]
         line["roofline"] = {"bound": "hbm", "achieved": k["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",

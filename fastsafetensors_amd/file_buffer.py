@@ -145,8 +145,23 @@ class FilesBufferOnDevice:
     def as_dict(self, tensor_shard_dim: "OrderedDict[str, int]") -> Dict[str, TensorBase]:
         """``{name: dim}`` -> ``{name: tensor}`` with the rule of ``get_sharded``."""
         out: Dict[str, TensorBase] = {}
+        run: List[Tuple[str, int]] = []  # consecutive names that live in the same file
+        run_of: Optional[Tuple[int, int]] = None
+
+        def flush() -> None:
+            if not run:
+                return
+            rank, lidx = run_of
+            out.update(self.rank_loaders[rank][lidx].shuffle_many(self.pg, run))
+            for name, _ in run:
+                self._mark_used(rank, lidx, name)
+            run.clear()
+
         for name, dim in tensor_shard_dim.items():
-            rank, lidx, factory = self._factory(name)
-            out[name] = factory.shuffle(self.pg, name, dim)
-            self._mark_used(rank, lidx, name)
-        return out
+            where = self._get_rank_lidx(name)
+            if where != run_of:
+                flush()
+                run_of = where
+            run.append((name, dim))
+        flush()
+        return {name: out[name] for name in tensor_shard_dim}

@@ -118,6 +118,13 @@ class FrameworkOpBase(ABC):
     ) -> TensorBase:
         """Dense copy of rank ``rank``'s ``ceil(S/world)`` block of ``src`` along ``dim``."""
 
+    def extract_shards(self, items: List[Tuple[TensorBase, Any, int]], rank: int, world: int) -> List[TensorBase]:
+        """Many ``extract_shard`` calls at once; ``dim == -1`` means a copy of the whole tensor."""
+        return [
+            src.clone().detach() if dim == -1 else self.extract_shard(src, frame, dim, rank, world)
+            for src, frame, dim in items
+        ]
+
     def get_storage_shape(
         self, dtype: DType, shape: List[int], strides: List[int]
     ) -> Tuple[List[int], List[int]]:

@@ -321,6 +321,31 @@ class TorchOp(FrameworkOpBase):
             _native.slice_copy(dst.data_ptr(), src.data_ptr() + first, outer, seg, pitch, stream)
         return dst
 
+    def extract_shards(
+        self, items: List[Tuple[TorchTensor, TensorFrame, int]], rank: int, world: int
+    ) -> List[TorchTensor]:
+        """``extract_shard`` for many tensors with batched launches; ``dim == -1``
+        asks for a private copy of the whole tensor."""
+        outs: List[TorchTensor] = []
+        jobs = []
+        stream = None
+        for src, frame, dim in items:
+            if dim == -1:
+                out_shape, outer, seg, pitch, first = list(frame.shape), 1, frame.nbytes, frame.nbytes, 0
+            else:
+                out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world)
+            dst = self.get_empty_tensor(out_shape, frame.dtype, src.device)
+            outs.append(dst)
+            if outer * seg:
+                if not src.real_tensor.is_cuda:
+                    raise RuntimeError("extract_shards needs tensors in GPU memory (no CPU path exists)")
+                if stream is None:
+                    stream = torch.cuda.current_stream(src.real_tensor.device).cuda_stream
+                jobs.append((dst.data_ptr(), src.data_ptr() + first, outer, seg, pitch))
+        if jobs:
+            _native.slice_copy_batch(jobs, stream)
+        return outs
+
     # ---- misc ------------------------------------------------------------------
     def synchronize(self, device: Device) -> None:
         if device.type != DeviceType.CPU and torch.cuda.is_available():

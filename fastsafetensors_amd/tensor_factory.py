@@ -132,6 +132,34 @@ class LazyTensorFactory:
             self.shuffled[tensor_name] = out
         return out
 
+    def shuffle_many(self, pg: ProcessGroupBase, names_dims: List[Tuple[str, int]]) -> Dict[str, TensorBase]:
+        """``shuffle`` for many tensors of this file at once: the copies of all of
+        them go to the GPU as batched launches instead of one launch per tensor."""
+        if pg.size() == 1:
+            return {name: self.tensors[name] for name, _ in names_dims}
+        out: Dict[str, TensorBase] = {}
+        todo: List[Tuple[str, int]] = []
+        for name, dim in names_dims:
+            if name in self.shuffled:
+                out[name] = self.shuffled[name].clone().detach()
+            else:
+                if self.rank != pg.rank():
+                    self._no_peer("shuffle", name)
+                todo.append((name, dim))
+        made = self.framework.extract_shards(
+            [(self._held(name, "shuffle"), self.metadata.tensors[name], dim) for name, dim in todo],
+            pg.rank(), pg.size(),
+        )
+        for (name, dim), t in zip(todo, made):
+            if dim == -1:
+                pg.broadcast(t, self.rank)
+            else:
+                pg.scatter(t, scatter_list=[], src=self.rank)
+            if not self.disable_cache:
+                self.shuffled[name] = t
+            out[name] = t
+        return out
+
     def shuffle_multi_cols(self, pg: ProcessGroupBase, tensor_names: List[str], dim: int) -> TensorBase:
         """The rank's blocks of several tensors joined along ``dim``
         (``tensor_factory.py:194-259``)."""
