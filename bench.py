@@ -349,6 +349,31 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     del srcs, keep, launches
     torch.cuda.empty_cache()
 
+    # -- slice extract on shapes whose rows are not multiples of 16 bytes: the LDS-staged
+    #    kernel against the direct kernel at the small unit such shapes force
+    odd = {}
+    for label, shape, tdt in [("bf16 [11008, 4090] cut in 4 along dim 1 (2046-byte segments, 8180-byte pitch)", (11008, 4090), torch.int16),
+                              ("fp8 [8192, 8190] cut in 4 along dim 1 (2048-byte segments, 8190-byte pitch)", (8192, 8190), torch.uint8)]:
+        t = torch.randint(0, 100, shape, dtype=tdt, device=dev)
+        item = t.element_size()
+        block = -(-shape[1] // world)
+        dsts = [torch.empty((shape[0], min(block, shape[1] - r * block)), dtype=tdt, device=dev) for r in range(world)]
+        jobs = [(dsts[r].data_ptr(), t.data_ptr() + r * block * item, shape[0], dsts[r].shape[1] * item, shape[1] * item)
+                for r in range(world)]
+        nb = 2 * sum(d.numel() * item for d in dsts)
+        res = {}
+        for mode, env in (("lds_staged", "0"), ("direct_small_unit", "1")):
+            os.environ["FSTX_NO_LDS_SLICE"] = env
+            _native.slice_copy_batch(jobs, stream)
+            ms = timed([lambda: _native.slice_copy_batch(jobs, stream)] * 5)
+            res[mode] = {"avg_launch_ms": sum(ms) / len(ms), "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
+            if not all(torch.equal(dsts[r], t[:, r * block : (r + 1) * block]) for r in range(world)):
+                raise SystemExit(f"bench: odd-shape slice ({mode}) differs from torch's slice")
+        os.environ.pop("FSTX_NO_LDS_SLICE")
+        odd[label] = dict(res, bytes_per_launch=nb)
+        del t, dsts
+    out["slice_extract_odd_shapes"] = odd
+
     # -- realign: config C2's data section shifted by header_length % 16 = 10 bytes
     n = 709_646_336
     cal = 1 << 30

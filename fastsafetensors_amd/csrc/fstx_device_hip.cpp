@@ -7,6 +7,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "fstx.h"
 #include "fstx_internal.h"
 
@@ -97,4 +99,8 @@ int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stre
 
 namespace fstx_internal {
 int check_launch(const char *what) { return rc(hipGetLastError(), what); }
+bool lds_path_disabled() {
+    const char *e = getenv("FSTX_NO_LDS_SLICE"); // read per call so that a benchmark can flip it
+    return e && e[0] == '1';
+}
 } // namespace fstx_internal

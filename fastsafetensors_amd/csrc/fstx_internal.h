@@ -38,6 +38,7 @@ int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stre
 namespace fstx_internal {
 
 int check_launch(const char *what);  // hipGetLastError -> 0 / -FSTX_E_HIP
+bool lds_path_disabled();            // FSTX_NO_LDS_SLICE=1: odd-aligned slices stay on the direct kernel (measurements)
 bool debug_enabled();
 void debug(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 void note_bounce_bytes(int64_t delta); // process-wide pinned ring accounting

@@ -227,6 +227,148 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     }
 }
 
+// ------------------------------------- slice extract, staged through LDS
+//
+// For segments whose length, pitch or source address is not a multiple of 16
+// bytes the direct kernel above has to drop to 8-, 4-, 2- or 1-byte moves per
+// lane.  This variant keeps every global access 16 bytes wide: a wavefront owns
+// a 4 KiB tile of the (16-byte aligned) destination, loads the aligned 16-byte
+// source vectors that cover the tile's rows into LDS -- each row into its own
+// slot, at the same offset modulo 16 it has in memory -- and then assembles each
+// destination vector from naturally aligned `unit`-sized LDS reads.  The odd
+// alignment is absorbed by LDS, whose banks do not care about it.
+
+constexpr uint32_t kTileBytes = 4096; // destination bytes per wavefront
+constexpr uint32_t kLdsMinSeg = 64;   // shorter segments stay on the direct kernel
+// LDS slot of the tile's i-th row piece starts at align_down(s_i + 48 i, 16), where s_i is
+// the piece's position in the tile: consecutive slots then never overlap (a piece of L bytes
+// needs at most L + 30 bytes once both ends are widened to 16-byte vectors), and a tile
+// touches at most floor(4094 / 64) + 2 = 65 rows.
+constexpr uint32_t kRowGap = 48;
+constexpr uint32_t kLdsBytes = kTileBytes + kRowGap * 66 + 64;
+
+struct alignas(32) LdsSliceJob {
+    char *dst;            // 16-byte aligned
+    const char *src;
+    uint64_t pitch_unit;  // pitch (< 2^56) | log2(unit bytes) << 56
+    uint32_t seg_bytes;   // kLdsMinSeg <= seg_bytes
+    uint32_t outer;       // number of segments
+};
+
+template <int U> struct UnitOf;
+template <> struct UnitOf<1> { typedef uint8_t type; };
+template <> struct UnitOf<2> { typedef uint16_t type; };
+template <> struct UnitOf<4> { typedef uint32_t type; };
+template <> struct UnitOf<8> { typedef uint64_t type; };
+
+// geometry of one tile: which rows it touches and where each row piece sits
+struct TileGeom {
+    const char *src;
+    uint64_t pitch, d0, d1, row_first, row_last;
+    uint32_t seg, first_col;
+
+    __device__ __forceinline__ uint32_t col_begin(uint64_t row) const { return row == row_first ? first_col : 0; }
+    __device__ __forceinline__ uint32_t col_end(uint64_t row) const {
+        return row == row_last ? (uint32_t)(d1 - row_last * seg) : seg;
+    }
+    __device__ __forceinline__ uintptr_t src_begin(uint64_t row) const {
+        return (uintptr_t)src + row * pitch + col_begin(row);
+    }
+    // LDS offset of the 16-byte vector that holds the row piece's first source byte
+    __device__ __forceinline__ uint32_t slot(uint64_t row) const {
+        const uint32_t i = (uint32_t)(row - row_first);
+        const uint32_t s = i == 0 ? 0u : (uint32_t)(row * seg - d0);
+        return (s + kRowGap * i) & ~15u;
+    }
+};
+
+template <int U>
+__device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, unsigned char *lds) {
+    typedef typename UnitOf<U>::type unit_t;
+    const uint32_t lane = threadIdx.x;
+    TileGeom g;
+    g.src = job.src;
+    g.pitch = job.pitch_unit & 0x00ffffffffffffffull;
+    g.seg = job.seg_bytes;
+    const uint64_t total = (uint64_t)job.outer * g.seg;
+    g.d0 = (uint64_t)tile * kTileBytes;
+    g.d1 = g.d0 + kTileBytes < total ? g.d0 + kTileBytes : total;
+    g.row_first = g.d0 / g.seg;
+    g.row_last = (g.d1 - 1) / g.seg;
+    g.first_col = (uint32_t)(g.d0 - g.row_first * g.seg);
+    const uint32_t nrows = (uint32_t)(g.row_last - g.row_first) + 1;
+
+    // ---- phase 1: aligned 16-byte loads.  `group` lanes share a row piece; short rows are
+    // loaded several per step so that the lanes stay busy.
+    const uint32_t longest = g.seg < kTileBytes ? g.seg : kTileBytes;
+    const uint32_t vmax = (longest + 30) / 16 + 1; // vectors a row piece can need
+    uint32_t group = 64;
+    while (group / 2 >= vmax) group /= 2;
+    const uint32_t rows_per_step = 64 / group;
+    for (uint32_t ibase = 0; ibase < nrows; ibase += rows_per_step) {
+        const uint32_t i = ibase + lane / group;
+        if (i < nrows) {
+            const uint64_t row = g.row_first + i;
+            const uintptr_t a0 = g.src_begin(row), a1 = a0 + (g.col_end(row) - g.col_begin(row));
+            const uintptr_t lo = a0 & ~(uintptr_t)15;
+            const uint32_t at = g.slot(row);
+            for (uint32_t v = lane % group; lo + 16ull * v < a1; v += group)
+                *reinterpret_cast<v4u *>(lds + at + 16 * v) =
+                    __builtin_nontemporal_load(reinterpret_cast<const v4u *>(lo) + v);
+        }
+    }
+    __syncthreads(); // one wavefront: orders its LDS writes before the reads below
+
+    // ---- phase 2: every lane assembles its destination vectors from LDS
+    for (uint64_t d = g.d0 + 16ull * lane; d < g.d1; d += 16 * 64) {
+        uint64_t row = d / g.seg;
+        uint32_t col = (uint32_t)(d - row * g.seg);
+        // LDS address of column `col` of `row` = bias + col
+        auto bias_of = [&](uint64_t r) -> int32_t {
+            return (int32_t)(g.slot(r) + ((uint32_t)g.src_begin(r) & 15u)) - (int32_t)g.col_begin(r);
+        };
+        int32_t bias = bias_of(row);
+        const uint32_t nbytes = g.d1 - d < 16 ? (uint32_t)(g.d1 - d) : 16u;
+        unit_t piece[16 / U];
+#pragma unroll
+        for (int p = 0; p < 16 / U; ++p) {
+            piece[p] = 0;
+            if ((uint32_t)p * U < nbytes) {
+                piece[p] = *reinterpret_cast<const unit_t *>(lds + (bias + (int32_t)col));
+                col += U;
+                if (col >= g.seg) {
+                    col = 0;
+                    ++row;
+                    if (row <= g.row_last) bias = bias_of(row);
+                }
+            }
+        }
+        if (nbytes == 16) {
+            v4u out;
+            __builtin_memcpy(&out, piece, 16);
+            __builtin_nontemporal_store(out, reinterpret_cast<v4u *>(job.dst + d));
+        } else { // the job's last, partial vector
+            for (uint32_t p = 0; p * U < nbytes; ++p) reinterpret_cast<unit_t *>(job.dst + d)[p] = piece[p];
+        }
+    }
+}
+
+__global__ __launch_bounds__(64) void slice_lds_kernel(const uint32_t granule_log2,
+                                                       const JobTable<LdsSliceJob> t) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[kLdsBytes];
+    const uint32_t b = blockIdx.x;
+    const uint32_t ji = find_job(t, granule_log2, b);
+    const LdsSliceJob job = t.fetch(ji);
+    const uint32_t tile = b - t.first_block[ji];
+    if ((uint64_t)tile * kTileBytes >= (uint64_t)job.outer * job.seg_bytes) return; // idle granule padding
+    switch ((uint32_t)(job.pitch_unit >> 56)) { // uniform across the workgroup
+    case 3: lds_tile<8>(job, tile, lds); break;
+    case 2: lds_tile<4>(job, tile, lds); break;
+    case 1: lds_tile<2>(job, tile, lds); break;
+    default: lds_tile<1>(job, tile, lds); break;
+    }
+}
+
 // --------------------------------------------------------------- host side
 
 inline uint32_t blocks_for(uint64_t items) {
@@ -294,9 +436,20 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     if (!descs) return -FSTX_E_INVAL;
     if (n > FSTX_BATCH_MAX) return -FSTX_E_TOO_MANY;
     JobTable<SliceJob> t;
-    uint64_t blocks_of[FSTX_BATCH_MAX];
-    uint64_t blocks = 0;
-    uint32_t k = 0;
+    JobTable<LdsSliceJob> tl;
+    uint64_t blocks_of[FSTX_BATCH_MAX], tiles_of[FSTX_BATCH_MAX];
+    uint64_t blocks = 0, tiles = 0;
+    uint32_t k = 0, kl = 0;
+    auto flush_lds = [&]() -> int {
+        if (kl == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t grid = plan_grid(tl, tiles_of, kl, &gl);
+        hipLaunchKernelGGL(slice_lds_kernel, dim3((uint32_t)grid), dim3(64), 0,
+                           static_cast<hipStream_t>(stream), gl, tl);
+        kl = 0;
+        tiles = 0;
+        return fstx_internal::check_launch("slice_lds_kernel");
+    };
     auto flush = [&]() -> int {
         if (k == 0) return 0;
         uint32_t gl = 0;
@@ -323,6 +476,21 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         uint64_t outer = d.outer, seg = d.seg_bytes, pitch = d.src_pitch;
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src |
                                              seg | pitch | 16u);
+        if (ul < 4 && seg >= kLdsMinSeg && seg <= 0xffffffffull && outer <= 0xffffffffull &&
+            ((uintptr_t)d.dst & 15) == 0 && !fstx_internal::lds_path_disabled()) {
+            // odd alignment somewhere: keep the global accesses 16 bytes wide and realign through LDS
+            const uint64_t n_tiles = (outer * seg + kTileBytes - 1) / kTileBytes;
+            if (kl == FSTX_BATCH_MAX || tiles + n_tiles > kMaxBlocksPerLaunch) {
+                int rc = flush_lds();
+                if (rc < 0) return rc;
+            }
+            tl.job[kl] = LdsSliceJob{static_cast<char *>(d.dst), static_cast<const char *>(d.src),
+                                     pitch | ((uint64_t)ul << 56), (uint32_t)seg, (uint32_t)outer};
+            tiles_of[kl] = n_tiles;
+            tiles += n_tiles;
+            ++kl;
+            continue;
+        }
         const uint64_t seg_units = seg >> ul;
         // rows per job so that the unit index fits 32 bits
         uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
@@ -344,6 +512,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     }
     int rc = flush();
     if (rc < 0) return rc;
+    if ((rc = flush_lds()) < 0) return rc;
     return n_spans ? fstx_realign_copy_batch(spans, n_spans, stream) : 0;
 }
 

@@ -190,6 +190,41 @@ def test_slice_batch_and_round_trip_full_size_c4(dev):
             assert torch.equal(parts[rank].view(torch.int16), t[sl].contiguous().view(torch.int16))
 
 
+def test_slice_odd_shapes_go_through_lds(dev):
+    """Segments that are not multiples of 16 bytes (odd column counts, 1-byte dtypes,
+    shifted sources): the LDS-staged kernel, against torch's own slicing on the GPU,
+    and against the direct small-unit kernel (FSTX_NO_LDS_SLICE=1)."""
+    import os
+
+    rng = np.random.default_rng(11)
+    cases = [((4096, 1000), torch.int16, 1, 4), ((3000, 999), torch.uint8, 1, 3), ((257, 4094), torch.uint8, 1, 2),
+             ((129, 2047), torch.uint8, 1, 1), ((64, 65, 33), torch.int16, 1, 5), ((1000, 250), torch.int32, 1, 2),
+             ((31, 8190), torch.int16, 1, 2), ((5, 100_003), torch.uint8, 1, 4), ((2000, 130), torch.uint8, 1, 2)]
+    for shape, dtype, dim, world in cases:
+        item = torch.empty((), dtype=dtype).element_size()
+        hi = 127 if dtype == torch.uint8 else 30000
+        for shift in (0, item, 3 * item):
+            base = torch.randint(0, hi, (int(np.prod(shape)) + 64,), dtype=dtype, device=dev)
+            t = base[shift // item : shift // item + int(np.prod(shape))].view(shape)
+            for rank in range(world):
+                block = -(-shape[dim] // world)
+                lo, hi_ = min(rank * block, shape[dim]), min((rank + 1) * block, shape[dim])
+                want = t[(slice(None),) * dim + (slice(lo, hi_),)].contiguous()
+                inner = int(np.prod(shape[dim + 1 :], dtype=np.int64)) * item
+                outer = int(np.prod(shape[:dim], dtype=np.int64))
+                outs = []
+                for no_lds in ("0", "1"):
+                    os.environ["FSTX_NO_LDS_SLICE"] = no_lds
+                    got = torch.full((want.numel() + 32,), 77, dtype=dtype, device=dev)
+                    _native.slice_copy(got.data_ptr() + 16 * item * 0 + 0, t.data_ptr() + lo * inner, outer,
+                                       (hi_ - lo) * inner, shape[dim] * inner, stream())
+                    outs.append(got)
+                os.environ.pop("FSTX_NO_LDS_SLICE")
+                for got in outs:
+                    assert torch.equal(got[: want.numel()].view(want.shape), want), (shape, dtype, rank, shift)
+                    assert (got[want.numel() :] == 77).all(), "wrote past the end of the shard"
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
