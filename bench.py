@@ -176,15 +176,9 @@ def measure_h2d_peak(gib: int = 4, chunk: int = 16 << 20, streams: int = 2) -> f
 
 
 def checksum(t) -> Tuple[int, int]:
-    """Order-sensitive 64-bit check words of a tensor's bytes, computed on its device."""
-    import torch
+    from fastsafetensors_amd.checkpoints import tensor_checksum
 
-    b = t.contiguous().reshape(-1).view(torch.uint8)
-    n4 = b.numel() // 4 * 4
-    w = b[:n4].view(torch.int32).to(torch.int64)
-    idx = torch.arange(w.numel(), device=w.device, dtype=torch.int64) % 8191 + 1
-    tail = int(b[n4:].to(torch.int64).sum().item()) if n4 < b.numel() else 0
-    return int(w.sum().item()) + tail, int((w * idx).sum().item())
+    return tensor_checksum(t)
 
 
 def run_load(files: List[str], read_mode: str, threads: int, block_kb: int, verify=None) -> Dict[str, float]:

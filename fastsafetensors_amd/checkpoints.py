@@ -170,6 +170,18 @@ def write_checkpoint(
             "specs": ordered}
 
 
+def tensor_checksum(t: torch.Tensor) -> Tuple[int, int]:
+    """Two order-sensitive 64-bit check words of a tensor's bytes, computed on the
+    tensor's device: the sum of its 32-bit words and the sum of those words weighted
+    by their position (mod 8191).  A shifted, swapped or stale region changes them."""
+    b = t.contiguous().reshape(-1).view(torch.uint8)
+    n4 = b.numel() // 4 * 4
+    w = b[:n4].view(torch.int32).to(torch.int64)
+    idx = torch.arange(w.numel(), device=w.device, dtype=torch.int64) % 8191 + 1
+    tail = int(b[n4:].to(torch.int64).sum().item()) if n4 < b.numel() else 0
+    return int(w.sum().item()) + tail, int((w * idx).sum().item())
+
+
 class _NoDigest:
     def update(self, _b) -> None:
         pass
