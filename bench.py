@@ -42,6 +42,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one launch of the roofline workload (slice_kernel, C4 column cuts, 28 tensors) moved
+# according to rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by its reading for an aligned
+# 1 GiB copy (x1.99988 and x0.99965): profiles/fstx_kernels_hbm_traffic_counters.md.  Algorithmic:
+# 1,357,905,920.
+SLICE_KERNEL_TRAFFIC_BYTES = 1_357_731_888
 
 
 def log(*a):
@@ -292,15 +297,18 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         torch.cuda.synchronize()
         return [a.elapsed_time(b) for a, b in evs]
 
-    # -- slice extract: one third of config C4 (14 of 40 layers + embeddings), TP=4
+    # -- config C4 (Llama-2-13B, TP=4), the tensors of file 1 of 3 resident in HBM, every rank in turn.
+    #    Column cuts (o_proj, down_proj: dim 1) are strided gathers -> slice_kernel, one launch of 28
+    #    tensors per rank.  Row cuts (q/k/v/gate/up/embed: dim 0) are contiguous spans -> the same
+    #    entry point hands them to realign_kernel as plain copies, two launches of <= 48 per rank.
     world = 4
     specs = [s for s in ck.configs(1.0)["C4"].files()[0] if ck.llama_shard_dim(s.name) >= 0]
     g = torch.Generator(device=dev).manual_seed(1)
     srcs = {s.name: torch.randint(-32768, 32767, s.shape, dtype=torch.int16, device=dev, generator=g) for s in specs}
-    launches = []  # (jobs, algorithmic bytes)
-    keep = []
+    keep = {}
+    launches = {0: [], 1: []}  # cut dim -> [(jobs, algorithmic bytes)]
     for rank in range(world):
-        jobs = []
+        jobs = {0: [], 1: []}
         for s in specs:
             dim = ck.llama_shard_dim(s.name)
             block = -(-s.shape[dim] // world)
@@ -309,37 +317,44 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
             out_shape = list(s.shape)
             out_shape[dim] = block
             dst = torch.empty(out_shape, dtype=torch.int16, device=dev)
-            keep.append(dst)
-            jobs.append((dst.data_ptr(), srcs[s.name].data_ptr() + rank * block * inner, outer, block * inner,
-                         s.shape[dim] * inner))
-        for i in range(0, len(jobs), _native.FSTX_BATCH_MAX):
-            part = jobs[i : i + _native.FSTX_BATCH_MAX]
-            launches.append((part, 2 * sum(j[2] * j[3] for j in part)))
-    for _ in range(max(1, warmup)):
-        for part, _b in launches:
-            _native.slice_copy_batch(part, stream)
-    times, nbytes, pass_ms = [], [], []
-    for _ in range(max(1, steps)):
-        times += timed([lambda p=part: _native.slice_copy_batch(p, stream) for part, _b in launches])
-        nbytes += [b for _p, b in launches]
-        # the same launches between ONE pair of events: no marker between kernels
-        pass_ms += timed([lambda: [_native.slice_copy_batch(p, stream) for p, _b in launches]])
+            keep[(s.name, rank)] = dst
+            jobs[dim].append((dst.data_ptr(), srcs[s.name].data_ptr() + rank * block * inner, outer, block * inner,
+                              s.shape[dim] * inner))
+        for dim in (0, 1):
+            for i in range(0, len(jobs[dim]), _native.FSTX_BATCH_MAX):
+                part = jobs[dim][i : i + _native.FSTX_BATCH_MAX]
+                launches[dim].append((part, 2 * sum(j[2] * j[3] for j in part)))
+
+    def measure(group, label):
+        for _ in range(max(1, warmup)):
+            for part, _b in group:
+                _native.slice_copy_batch(part, stream)
+        times, nbytes, pass_ms = [], [], []
+        for _ in range(max(1, steps)):
+            times += timed([lambda p=part: _native.slice_copy_batch(p, stream) for part, _b in group])
+            nbytes += [b for _p, b in group]
+            # the same launches between ONE pair of events: no marker between kernels
+            pass_ms += timed([lambda: [_native.slice_copy_batch(p, stream) for p, _b in group]])
+        avg_ms = sum(pass_ms) / len(pass_ms) / len(group)
+        avg_b = sum(nbytes) / len(nbytes)
+        return {"workload": label, "launches_timed": len(pass_ms) * len(group), "avg_launch_ms": avg_ms,
+                "bytes_per_launch": avg_b, "achieved_GBps": avg_b / 1e6 / avg_ms,
+                "best_GBps": max(b / 1e6 / t for b, t in zip(nbytes, times)),
+                "avg_launch_ms_with_event_markers": sum(times) / len(times)}
+
+    n1 = sum(1 for s in specs if ck.llama_shard_dim(s.name) == 1)
+    out["slice_extract"] = measure(
+        launches[1], f"C4 Llama-2-13B bf16 TP=4, column cuts of file 1 of 3: {n1} tensors (o_proj 2,560-byte segments at "
+                     f"pitch 10,240; down_proj 6,912 at 27,648) per launch, one launch per rank (slice_kernel)")
+    out["row_block_copy"] = measure(
+        launches[0], f"C4 Llama-2-13B bf16 TP=4, row cuts of file 1 of 3: {len(specs) - n1} tensors per rank in "
+                     f"{len(launches[0]) // world} launches (contiguous spans, realign_kernel without shift)")
     # parity at full size: the four ranks' blocks put side by side give the tensor back
-    per_rank = len(specs)
-    for i, s in enumerate(specs):
+    for s in specs:
         dim = ck.llama_shard_dim(s.name)
-        whole = torch.cat([keep[r * per_rank + i] for r in range(world)], dim=dim)
+        whole = torch.cat([keep[(s.name, r)] for r in range(world)], dim=dim)
         if not torch.equal(whole, srcs[s.name]):
             raise SystemExit(f"bench: shards of {s.name} do not concatenate back to the tensor")
-    avg_ms = sum(pass_ms) / len(pass_ms) / len(launches)
-    avg_b = sum(nbytes) / len(nbytes)
-    out["slice_extract"] = {
-        "workload": f"C4 Llama-2-13B bf16 TP=4, file 1 of 3: {len(specs)} sharded tensors x 4 ranks, "
-                    f"{len(launches)} launches of <= {_native.FSTX_BATCH_MAX} tensors",
-        "launches_timed": len(pass_ms) * len(launches), "avg_launch_ms": avg_ms, "bytes_per_launch": avg_b,
-        "achieved_GBps": avg_b / 1e6 / avg_ms, "best_GBps": max(b / 1e6 / t for b, t in zip(nbytes, times)),
-        "avg_launch_ms_with_event_markers": sum(times) / len(times),
-    }
     del srcs, keep, launches
     torch.cuda.empty_cache()
 
@@ -623,7 +638,8 @@ def main() -> None:
     if kernels:
         k = kernels["slice_extract"]
         line["roofline"] = {"bound": "hbm", "achieved": k["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                            "frac": k["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": "slice_kernel",
+                            "frac": k["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": SLICE_KERNEL_TRAFFIC_BYTES,
+                            "kernel": "slice_kernel",
                             "workload": k["workload"], "avg_launch_ms": k["avg_launch_ms"],
                             "bytes_per_launch": k["bytes_per_launch"]}
         line["kernels"] = kernels
