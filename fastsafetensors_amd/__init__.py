@@ -7,6 +7,7 @@ from .common import SafeTensorsMetadata, SingleGroup, TensorFrame, get_device_nu
 from .file_buffer import FilesBufferOnDevice
 from .frameworks._torch import StubProcessGroup
 from .loader import BaseSafeTensorsFileLoader, SafeTensorsFileLoader, fastsafe_open
+from .parallel_loader import ParallelLoader, PipelineParallel
 from .st_types import Device, DeviceType, DType
 
 __all__ = [
@@ -15,6 +16,8 @@ __all__ = [
     "DeviceType",
     "DType",
     "FilesBufferOnDevice",
+    "ParallelLoader",
+    "PipelineParallel",
     "SafeTensorsFileLoader",
     "SafeTensorsMetadata",
     "SingleGroup",

@@ -94,6 +94,10 @@ class MI355XFileCopier(CopierInterface):
         total = meta.size_bytes - first
         lead = self.data_at if self.layout == "direct" else 0
         gbuf = self.framework.alloc_tensor_memory(lead + total, self.device)
+        # The allocator may hand back memory that kernels already queued on the caller's
+        # stream still read (a buffer closed a moment ago).  The copy streams are not
+        # ordered after that stream, so let it drain before they write into the arena.
+        self.framework.synchronize(self.device)
         try:
             done = 0
             while done < total:

@@ -18,6 +18,7 @@ dtype table (``:17-49``), tensor wrapper (``:52-98``), process group wrapper
 """
 
 import math
+import threading
 from dataclasses import dataclass
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
@@ -148,6 +149,11 @@ class StubProcessGroup(TorchProcessGroup):
 class TorchOp(FrameworkOpBase):
     def __init__(self) -> None:
         self.mem_used = 0
+        self._mem_lock = threading.Lock()  # a producer thread allocates while the caller frees
+
+    def _account(self, delta: int) -> None:
+        with self._mem_lock:
+            self.mem_used += delta
 
     def get_name(self) -> str:
         return "pytorch"
@@ -163,17 +169,17 @@ class TorchOp(FrameworkOpBase):
     # ---- memory ------------------------------------------------------------
     def alloc_tensor_memory(self, length: int, dev: Device) -> _native.DeviceBuffer:
         arena = torch.empty(max(length, 1), dtype=torch.uint8, device=dev.as_str())
-        self.mem_used += length
+        self._account(length)
         return _native.DeviceBuffer(arena.data_ptr(), length, dev.type != DeviceType.CPU, arena)
 
     def free_tensor_memory(self, gbuf: _native.DeviceBuffer, dev: Device) -> None:
-        self.mem_used -= gbuf.total_length()
+        self._account(-gbuf.total_length())
         gbuf.extras.clear()
         gbuf.keepalive = None
 
     def shrink_tensor_memory(self, gbuf: _native.DeviceBuffer) -> None:
         """Give back the main allocation of ``gbuf`` but keep its side allocations."""
-        self.mem_used -= gbuf.get_length()
+        self._account(-gbuf.get_length())
         gbuf.keepalive = None
         gbuf._base, gbuf._length = 0, 0
 

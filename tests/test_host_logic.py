@@ -232,3 +232,64 @@ def test_shard_geometry_matches_oracle_shapes():
                     out_shape, outer, seg, pitch, first = FW.shard_geometry(frame, dim, rank, world)
                     assert out_shape == want_shape
                     assert outer * seg == int(np.prod(want_shape)) * bits // 8
+
+
+# ---- iterate_weights (producer / consumer) on the CPU ------------------------------------------
+
+
+def _tiny_files(tmp_path, n):
+    out, want = [], {}
+    for i in range(n):
+        p = str(tmp_path / f"part{i}.safetensors")
+        tensors = {f"f{i}.w{k}": torch.randn(3 + k, 5) for k in range(4)}
+        save_file(tensors, p)
+        out.append(p)
+        want.update(tensors)
+    return out, want
+
+
+@pytest.mark.parametrize("queue_size", [-1, 0, 2])
+def test_iterate_weights_streams_every_tensor(tmp_path, queue_size):
+    from fastsafetensors_amd import PipelineParallel
+
+    files, want = _tiny_files(tmp_path, 5)
+    loader = loader_for(None)
+    it = PipelineParallel(None, loader, files, queue_size=queue_size)
+    got = {}
+    live_after_close = []
+    for key, t in it.iterate_weights():
+        assert key not in got
+        got[key] = t
+        live_after_close.append(t)
+    assert list(got) == [k for i in range(5) for k in sorted(want) if k.startswith(f"f{i}.")]
+    for key, t in got.items():  # tensors outlive their batches: they are copies
+        assert torch.equal(t, want[key])
+    it.close()
+    assert FW.get_mem_used() == 0
+
+
+def test_iterate_weights_reports_producer_errors_and_cleans_up(tmp_path):
+    from fastsafetensors_amd import PipelineParallel
+
+    files, want = _tiny_files(tmp_path, 3)
+    files.insert(2, str(tmp_path / "missing.safetensors"))
+    it = PipelineParallel(None, loader_for(None), files, queue_size=0)
+    seen = []
+    with pytest.raises(FileNotFoundError):
+        for key, t in it.iterate_weights():
+            seen.append(key)
+    assert len(seen) == 8  # the two good files in front of the missing one
+    it.close()
+    assert FW.get_mem_used() == 0
+    # stopping early releases what the producer had already loaded
+    files, want = _tiny_files(tmp_path, 4)
+    it = PipelineParallel(None, loader_for(None), files, queue_size=3)
+    gen = it.iterate_weights()
+    next(gen)
+    gen.close()
+    it.close()
+    assert FW.get_mem_used() == 0
+    with pytest.raises(ValueError, match="max_concurrent_producers"):
+        PipelineParallel(None, loader_for(None), files, max_concurrent_producers=2)
+    with pytest.raises(NotImplementedError):
+        PipelineParallel(StubProcessGroup(0, 2), loader_for(StubProcessGroup(0, 2)), files)

@@ -290,3 +290,46 @@ def test_full_size_c1_and_c2(data_dir):
             loader.close()
         os.remove(path)
     assert_clean()
+
+
+@pytest.mark.parametrize("queue_size", [-1, 0, 2])
+def test_parallel_loader_iterate_weights(small_configs, queue_size):
+    """The vLLM-facing iterator: every tensor of every file once, in file order, as
+    copies that outlive their batch; byte-exact against the oracle's file bytes."""
+    from fastsafetensors_amd import ParallelLoader
+
+    files = small_configs["C5"]
+    it = ParallelLoader(None, files, queue_size=queue_size, device=DEV, max_threads=8)
+    got = {}
+    for key, t in it.iterate_weights():
+        assert key not in got and t.is_cuda and t.data_ptr() % 16 == 0
+        got[key] = t
+    it.close()
+    n = 0
+    for path in files:
+        h = orc.parse_file(path)
+        for name in h.tensors:
+            assert np.array_equal(dev_bytes(got[name]), orc.tensor_bytes(path, h, name)), name
+            n += 1
+    assert n == len(got)
+    got.clear()
+    assert_clean()
+
+
+def test_parallel_loader_error_and_early_stop(small_configs, tmp_path):
+    from fastsafetensors_amd import ParallelLoader
+
+    files = list(small_configs["C3"])
+    files.insert(2, str(tmp_path / "nope.safetensors"))
+    it = ParallelLoader(None, files, device=DEV, max_threads=4)
+    with pytest.raises(FileNotFoundError):
+        for _ in it.iterate_weights():
+            pass
+    it.close()
+    it = ParallelLoader(None, small_configs["C3"], queue_size=3, device=DEV, max_threads=4)
+    gen = it.iterate_weights()
+    first = next(gen)
+    gen.close()  # the consumer walks away after one tensor
+    it.close()
+    del first
+    assert_clean()
