@@ -125,6 +125,13 @@ class FrameworkOpBase(ABC):
             for src, frame, dim in items
         ]
 
+    def extract_shards_joined(
+        self, items: List[Tuple[TensorBase, Any]], dim: int, rank: int, world: int
+    ) -> Optional[TensorBase]:
+        """The rank's blocks of several tensors, written side by side along ``dim`` into one new
+        tensor by a single batched copy; ``None`` when the backend cannot place them directly."""
+        return None
+
     def get_storage_shape(
         self, dtype: DType, shape: List[int], strides: List[int]
     ) -> Tuple[List[int], List[int]]:

@@ -352,6 +352,27 @@ class TorchOp(FrameworkOpBase):
             _native.slice_copy_batch(jobs, stream)
         return outs
 
+    def extract_shards_joined(
+        self, items: List[Tuple[TorchTensor, TensorFrame]], dim: int, rank: int, world: int
+    ) -> Optional[TorchTensor]:
+        if not items or not all(src.real_tensor.is_cuda for src, _ in items):
+            return None
+        geoms = [self.shard_geometry(frame, dim, rank, world) for _, frame in items]
+        if any(g[1] != 1 for g in geoms):  # blocks are not contiguous in the joined tensor
+            return None
+        first_src, first_frame = items[0]
+        shape = list(geoms[0][0])
+        shape[dim] = sum(g[0][dim] for g in geoms)
+        out = self.get_empty_tensor(shape, first_frame.dtype, first_src.device)
+        jobs, at = [], out.data_ptr()
+        for (src, _), (_, outer, seg, pitch, first) in zip(items, geoms):
+            if seg:
+                jobs.append((at, src.data_ptr() + first, 1, seg, pitch))
+            at += seg
+        if jobs:
+            _native.slice_copy_batch(jobs, torch.cuda.current_stream(first_src.real_tensor.device).cuda_stream)
+        return out
+
     # ---- misc ------------------------------------------------------------------
     def synchronize(self, device: Device) -> None:
         if device.type != DeviceType.CPU and torch.cuda.is_available():

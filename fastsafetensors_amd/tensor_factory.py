@@ -162,8 +162,11 @@ class LazyTensorFactory:
 
     def shuffle_multi_cols(self, pg: ProcessGroupBase, tensor_names: List[str], dim: int) -> TensorBase:
         """The rank's blocks of several tensors joined along ``dim``
-        (``tensor_factory.py:194-259``)."""
-        pieces: List[TensorBase] = []
+        (``tensor_factory.py:194-259``).  The blocks are cut straight into their places in
+        the joined tensor by one batched launch when they are contiguous there (``dim``
+        is the outermost dimension with more than one entry); otherwise they are cut
+        first and concatenated afterwards."""
+        frames = []
         ref_shape: Optional[List[int]] = None
         for name in tensor_names:
             frame = self.metadata.tensors[name]
@@ -174,11 +177,15 @@ class LazyTensorFactory:
                     raise Exception(
                         f"dim {d} mismatch: tensor {name} has {frame.shape} vs. {ref_shape} (dim={dim})"
                     )
-            held = self._held(name, "shuffle_multi_cols")
-            if pg.size() == 1:
-                pieces.append(held)
-            else:
-                pieces.append(self.framework.extract_shard(held, frame, dim, pg.rank(), pg.size()))
+            frames.append(frame)
+        held = [self._held(name, "shuffle_multi_cols") for name in tensor_names]
+        rank, world = (0, 1) if pg.size() == 1 else (pg.rank(), pg.size())
+        joined = self.framework.extract_shards_joined(list(zip(held, frames)), dim, rank, world)
+        if joined is not None:
+            return joined
+        if pg.size() == 1:
+            return self.framework.concat_tensors(held, dim=dim)
+        pieces = self.framework.extract_shards([(h, f, dim) for h, f in zip(held, frames)], rank, world)
         return self.framework.concat_tensors(pieces, dim=dim)
 
     # -- release -----------------------------------------------------------------------

@@ -204,6 +204,12 @@ def test_as_dict_multi_cols_push_and_auto_free(small_configs):
     block = -(-refs[qkv[0]].shape[0] // world)
     want = torch.cat([refs[k][rank * block : (rank + 1) * block] for k in qkv], dim=0)
     assert torch.equal(joined.cpu().view(torch.int16), want.view(torch.int16))
+    # a join along dim 1 (column blocks side by side) takes the cut-then-concatenate route
+    o2 = [f"model.layers.{i}.self_attn.o_proj.weight" for i in (0, 1)]
+    joined = bufs.get_multi_cols(o2, dim=1).get_raw()
+    block = -(-refs[o2[0]].shape[1] // world)
+    want = torch.cat([refs[k][:, rank * block : (rank + 1) * block] for k in o2], dim=1)
+    assert torch.equal(joined.cpu().view(torch.int16), want.view(torch.int16))
     # push: a stub of rank 1 keeps what is pushed to rank 1, nothing otherwise
     pushed = bufs.push_tensor("model.norm.weight", 1)
     assert pushed is not None and torch.equal(pushed.cpu(), refs["model.norm.weight"])
