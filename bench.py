@@ -402,6 +402,24 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         "launches_timed": len(cal_times), "avg_launch_ms": sum(cal_times) / len(cal_times),
         "bytes_per_launch": 2 * cal, "achieved_GBps": 2 * cal / 1e6 / (sum(cal_times) / len(cal_times)),
     }
+    # -- down-cast on load: fp32 -> bf16 over 1 GiB of fp32 in 48 tensors per launch
+    #    (4 bytes read + 2 written per element)
+    per = cal // 4 // 48 // 16 * 16
+    src32 = window[: cal].view(torch.float32)
+    dst16 = dst[: cal // 2].view(torch.int16)
+    cjobs = [(dst16.data_ptr() + 2 * i * per, src32.data_ptr() + 4 * i * per, per,
+              _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"]) for i in range(48)]
+    _native.convert_batch(cjobs, stream)
+    conv_times = timed([lambda: _native.convert_batch(cjobs, stream)] * max(3, steps))
+    probe = slice(0, 1 << 22)
+    if not torch.equal(dst16[probe], src32[probe].to(torch.bfloat16).view(torch.int16)):
+        raise SystemExit("bench: converted values differ from torch's Tensor.to(bfloat16)")
+    conv_ms = sum(conv_times) / len(conv_times)
+    out["convert_f32_bf16"] = {
+        "workload": f"fp32 -> bf16, 48 tensors of {per} elements per launch (convert_kernel)",
+        "launches_timed": len(conv_times), "avg_launch_ms": conv_ms, "bytes_per_launch": 6 * per * 48,
+        "achieved_GBps": 6 * per * 48 / 1e6 / conv_ms,
+    }
     avg_ms = sum(times) / len(times)
     out["realign_copy"] = {
         "workload": "C2 GPT-2-medium fp16 data section, 709,646,336 bytes, source shifted by 10 bytes",

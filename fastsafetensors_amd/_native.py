@@ -80,6 +80,18 @@ class FstxSliceDesc(ctypes.Structure):
     ]
 
 
+class FstxConvertDesc(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("src", ctypes.c_void_p),
+        ("n_elems", ctypes.c_uint64),
+        ("src_type", ctypes.c_uint32),
+        ("dst_type", ctypes.c_uint32),
+    ]
+
+
+ELEM_TYPES = {"F64": 0, "F32": 1, "F16": 2, "BF16": 3, "F8_E4M3": 4, "F8_E5M2": 5}
+
 # name -> (restype, argtypes); must list every function include/fstx.h declares
 _SIGNATURES = {
     "fstx_abi_version": (ctypes.c_int, []),
@@ -114,6 +126,8 @@ _SIGNATURES = {
     ),
     "fstx_slice_copy_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxSliceDesc), ctypes.c_uint32, ctypes.c_void_p]),
+    "fstx_convert_batch": (
+        ctypes.c_int, [ctypes.POINTER(FstxConvertDesc), ctypes.c_uint32, ctypes.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -283,6 +297,14 @@ def slice_copy_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int
         part = jobs[i : i + FSTX_BATCH_MAX]
         arr = (FstxSliceDesc * len(part))(*[FstxSliceDesc(*j) for j in part])
         _check("fstx_slice_copy_batch", lib().fstx_slice_copy_batch(arr, len(part), stream))
+
+
+def convert_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:
+    """``jobs`` = (dst, src, n_elems, src_type, dst_type) tuples; any count."""
+    for i in range(0, len(jobs), FSTX_BATCH_MAX):
+        part = jobs[i : i + FSTX_BATCH_MAX]
+        arr = (FstxConvertDesc * len(part))(*[FstxConvertDesc(*j) for j in part])
+        _check("fstx_convert_batch", lib().fstx_convert_batch(arr, len(part), stream))
 
 
 # ---- reader ------------------------------------------------------------------------------

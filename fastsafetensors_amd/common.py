@@ -282,9 +282,9 @@ class SafeTensorsMetadata:
         ``gbuf`` byte 0 holds file byte ``copy_start_offset``; the view of a
         tensor therefore starts at ``header_length + s - copy_start_offset``.
         """
-        if dtype != DType.AUTO:
+        if dtype != DType.AUTO and any(f.dtype != dtype for f in self.tensors.values()):
             raise NotImplementedError(
-                "dtype conversion on load is outside this loader's scope; pass DType.AUTO"
+                "get_tensors builds views only; conversion on load is done by the copier (wait_io)"
             )
         shift = self.header_length - copy_start_offset
         return {

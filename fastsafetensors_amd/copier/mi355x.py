@@ -35,7 +35,7 @@ from typing import Dict, List, Optional, Tuple
 from .. import _native
 from ..common import SafeTensorsMetadata, TensorFrame
 from ..frameworks import FrameworkOpBase, TensorBase
-from ..st_types import Device, DeviceType, DType, dtype_storage_align
+from ..st_types import Device, DeviceType, DType, dtype_bits, dtype_storage_align
 from .base import CopierInterface
 from .registry import CopierConstructFunc, register_copier_constructor
 
@@ -135,12 +135,10 @@ class MI355XFileCopier(CopierInterface):
                 f"wait_io: read failed, file={self.metadata.src}, "
                 + ", ".join(f"req {r}: {e}" for r, e in failed)
             )
-        if dtype != DType.AUTO:
-            raise NotImplementedError(
-                "dtype conversion on load is outside this loader's scope; pass DType.AUTO"
-            )
         meta, fw = self.metadata, self.framework
         arena, data_at = gbuf, self.data_at
+        if dtype != DType.AUTO and any(f.dtype != dtype for f in meta.tensors.values()):
+            return self._converted(gbuf, dtype)
         if self.layout == "window" and not noalign and data_at % PTR_ALIGN and meta.data_length:
             # shift the whole data section onto a 16-byte boundary, out of place
             lead = pick_lead(list(meta.tensors.values()))
@@ -185,6 +183,62 @@ class MI355XFileCopier(CopierInterface):
                 tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
             else:
                 tensors[name] = fw.view_tensor(arena, data_at + frame.data_offsets[0], frame, self.device)
+        return tensors
+
+    def _converted(self, gbuf: _native.DeviceBuffer, dtype: DType) -> Dict[str, TensorBase]:
+        """Tensors down-cast to ``dtype`` on the GPU (``common.py:355-375`` does it with
+        ``Tensor.to`` + ``copy_`` per tensor): one batched kernel converts every tensor
+        that is not of ``dtype`` yet into a fresh arena; when nothing is left in the
+        original arena it goes back to the allocator, so the file ends up occupying
+        its converted size."""
+        meta, fw = self.metadata, self.framework
+        want_bits = dtype_bits(dtype)
+        src_at = gbuf.get_base_address() + self.data_at
+        placed: Dict[str, int] = {}
+        cursor = 0
+        for name, frame in meta.tensors.items():
+            if frame.dtype != dtype and frame.nbytes:
+                if want_bits > dtype_bits(frame.dtype):
+                    raise Exception(
+                        f"Online type conversion to larger sizes is not supported ({frame.dtype} -> {dtype})"
+                    )
+                if frame.dtype.value not in _native.ELEM_TYPES or dtype.value not in _native.ELEM_TYPES:
+                    raise NotImplementedError(
+                        f"conversion on load from {frame.dtype} to {dtype} has no kernel "
+                        f"(supported: {sorted(_native.ELEM_TYPES)})"
+                    )
+            if frame.dtype != dtype or (src_at + frame.data_offsets[0]) % PTR_ALIGN:
+                placed[name] = cursor
+                count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                cursor += _align_up(count * (want_bits if frame.dtype != dtype else dtype_bits(frame.dtype)) // 8, PTR_ALIGN)
+        side = fw.alloc_side_memory(gbuf, cursor, self.device)
+        convert, copy = [], []
+        for name, at in placed.items():
+            frame = meta.tensors[name]
+            src = src_at + frame.data_offsets[0]
+            if frame.dtype != dtype:
+                count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                if count:
+                    convert.append((side.get_base_address() + at, src, count,
+                                    _native.ELEM_TYPES[frame.dtype.value], _native.ELEM_TYPES[dtype.value]))
+            elif frame.nbytes:
+                copy.append((side.get_base_address() + at, src, frame.nbytes))
+        _native.convert_batch(convert, self._stream())
+        _native.realign_copy_batch(copy, self._stream())
+        fw.synchronize(self.device)
+        tensors: Dict[str, TensorBase] = {}
+        for name, frame in meta.tensors.items():
+            if name in placed:
+                if frame.dtype != dtype:
+                    count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                    frame = TensorFrame(dtype, frame.shape, [placed[name], placed[name] + count * want_bits // 8],
+                                        frame.strides, frame.offsets, frame.sliced)
+                    meta.tensors[name].dtype = dtype  # the header model reports the converted type from now on
+                tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
+            else:
+                tensors[name] = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)
+        if len(placed) == len(meta.tensors):
+            fw.shrink_tensor_memory(gbuf)  # nothing lives in the original arena any more
         return tensors
 
     def _stream(self) -> int:

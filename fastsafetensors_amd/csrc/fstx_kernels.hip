@@ -27,6 +27,19 @@ namespace {
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
+// Every pointer a job carries is device memory.  Saying so (address space 1) lets the
+// compiler emit global_load/global_store instead of flat accesses, which would have to
+// allow for LDS and scratch apertures and cannot be issued wide at odd alignments.
+#define FSTX_GLOBAL __attribute__((address_space(1)))
+template <typename T> __device__ __forceinline__ T ld_stream(const T *p) {
+    return __builtin_nontemporal_load((const FSTX_GLOBAL T *)p);
+}
+template <typename T> __device__ __forceinline__ void st_stream(T v, T *p) {
+    __builtin_nontemporal_store(v, (FSTX_GLOBAL T *)p);
+}
+template <typename T> __device__ __forceinline__ T ld_global(const T *p) { return *(const FSTX_GLOBAL T *)p; }
+template <typename T> __device__ __forceinline__ void st_global(T v, T *p) { *(FSTX_GLOBAL T *)p = v; }
+
 // One wavefront per workgroup measured fastest for a streaming copy on MI355X
 // (6.5 TB/s against 6.3 TB/s with 128..512 lanes): the dispatcher then spreads
 // single waves evenly and none waits for a sibling to retire.
@@ -145,7 +158,7 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
         const uint64_t e = threadIdx.x;
         if (e < edge) {
             const uint64_t at = e < head ? e : tail_at + (e - head);
-            job.dst[at] = job.src[at];
+            st_global(ld_global(job.src + at), job.dst + at);
         }
     }
 
@@ -156,7 +169,7 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
         // already aligned: a plain streaming copy, workgroups in dispatch order
         const uint64_t j = (uint64_t)lb * kBlock + threadIdx.x;
         const v4u *srcv = reinterpret_cast<const v4u *>(s);
-        if (j < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(srcv + j), dstv + j);
+        if (j < nvec) st_stream(ld_stream(srcv + j), dstv + j);
         return;
     }
     // Workgroups go round-robin over the eight dies, each with its own L2.  Give
@@ -177,8 +190,8 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     const v4u *srcv = reinterpret_cast<const v4u *>(s - m);
     const bool edge = live && ((threadIdx.x & 63) == 63 || j + 1 == nvec);
     v4u lo = {0, 0, 0, 0}, own_hi = {0, 0, 0, 0};
-    if (live) lo = __builtin_nontemporal_load(srcv + j);
-    if (edge) own_hi = __builtin_nontemporal_load(srcv + j + 1); // issued before lo is waited for
+    if (live) lo = ld_stream(srcv + j);
+    if (edge) own_hi = ld_stream(srcv + j + 1); // issued before lo is waited for
     v4u hi;
     hi.x = from_next_lane(lo.x);
     hi.y = from_next_lane(lo.y);
@@ -194,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     case 2: out = funnel<2>(lo, hi, r); break;
     default: out = funnel<3>(lo, hi, r); break;
     }
-    __builtin_nontemporal_store(out, dstv + j);
+    st_stream(out, dstv + j);
 }
 
 // ------------------------------------------------------------ slice extract
@@ -206,7 +219,7 @@ __device__ __forceinline__ void slice_units(const SliceJob &job, uint32_t u) {
     const uint64_t pitch = job.pitch_unit & 0x00ffffffffffffffull;
     const Unit *src = reinterpret_cast<const Unit *>(job.src + (uint64_t)row * pitch) + col;
     Unit *dst = reinterpret_cast<Unit *>(job.dst) + u;
-    __builtin_nontemporal_store(__builtin_nontemporal_load(src), dst);
+    st_stream(ld_stream(src), dst);
 }
 
 __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_log2,
@@ -313,8 +326,7 @@ __device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, 
             const uintptr_t lo = a0 & ~(uintptr_t)15;
             const uint32_t at = g.slot(row);
             for (uint32_t v = lane % group; lo + 16ull * v < a1; v += group)
-                *reinterpret_cast<v4u *>(lds + at + 16 * v) =
-                    __builtin_nontemporal_load(reinterpret_cast<const v4u *>(lo) + v);
+                *reinterpret_cast<v4u *>(lds + at + 16 * v) = ld_stream(reinterpret_cast<const v4u *>(lo) + v);
         }
     }
     __syncthreads(); // one wavefront: orders its LDS writes before the reads below
@@ -346,9 +358,9 @@ __device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, 
         if (nbytes == 16) {
             v4u out;
             __builtin_memcpy(&out, piece, 16);
-            __builtin_nontemporal_store(out, reinterpret_cast<v4u *>(job.dst + d));
+            st_stream(out, reinterpret_cast<v4u *>(job.dst + d));
         } else { // the job's last, partial vector
-            for (uint32_t p = 0; p * U < nbytes; ++p) reinterpret_cast<unit_t *>(job.dst + d)[p] = piece[p];
+            for (uint32_t p = 0; p * U < nbytes; ++p) st_global(piece[p], reinterpret_cast<unit_t *>(job.dst + d) + p);
         }
     }
 }
@@ -367,6 +379,163 @@ __global__ __launch_bounds__(64) void slice_lds_kernel(const uint32_t granule_lo
     case 1: lds_tile<2>(job, tile, lds); break;
     default: lds_tile<1>(job, tile, lds); break;
     }
+}
+
+// ------------------------------------------------- down-cast while loading
+//
+// copy_files_to_device(dtype=...) of the reference converts every tensor with
+// torch's Tensor.to() and copies the result back over the start of the tensor's
+// bytes (common.py:355-375).  Here one batched launch converts the tensors of a
+// file out of place into a smaller arena.  Rounding follows torch's own
+// conversions bit for bit: round to nearest even everywhere, bf16 NaNs become
+// 0x7fc0, fp8 e4m3fn has no infinity (everything from 480 up, and NaN, becomes
+// 0x7f), fp8 e5m2 overflows to infinity; double goes through float first.
+
+enum : uint32_t { kF64 = 0, kF32 = 1, kF16 = 2, kBF16 = 3, kF8E4M3 = 4, kF8E5M2 = 5 };
+
+struct alignas(32) ConvertJob {
+    char *dst;
+    const char *src;
+    uint64_t n_elems;
+    uint32_t src_type, dst_type;
+};
+
+__device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+template <uint32_t T> struct Elem;
+template <> struct Elem<kF64> {
+    typedef double type;
+    static __device__ __forceinline__ float to_f32(double v) {
+        // torch rounds double -> float -> target (two roundings).  The empty asm keeps the
+        // compiler from merging the two steps into one correctly rounded double -> half.
+        float f = (float)v;
+        asm volatile("" : "+v"(f));
+        return f;
+    }
+};
+template <> struct Elem<kF32> {
+    typedef float type;
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float f) { return f; }
+};
+template <> struct Elem<kF16> {
+    typedef _Float16 type;
+    static __device__ __forceinline__ float to_f32(_Float16 v) { return (float)v; }
+    static __device__ __forceinline__ _Float16 from_f32(float f) { return (_Float16)f; } // v_cvt_f16_f32: RNE
+};
+template <> struct Elem<kBF16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return bits_f32((uint32_t)v << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        const uint32_t u = f32_bits(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0; // NaN
+        return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    }
+};
+template <> struct Elem<kF8E4M3> {
+    typedef uint8_t type;
+    static __device__ __forceinline__ uint8_t from_f32(float f) {
+        uint32_t u = f32_bits(f);
+        const uint32_t sign = u & 0x80000000u;
+        u ^= sign;
+        uint8_t r;
+        if (u >= (1087u << 20)) {
+            r = 0x7f; // 480 and above, infinities and NaN
+        } else if (u < (121u << 23)) {
+            // below 2^-6, the smallest normal: let a float addition do the denormal rounding
+            const uint32_t magic = 141u << 23;
+            r = (uint8_t)(f32_bits(bits_f32(u) + bits_f32(magic)) - magic);
+        } else {
+            const uint32_t odd = (u >> 20) & 1u;
+            u += ((uint32_t)(7 - 127) << 23) + 0x7ffffu + odd;
+            r = (uint8_t)(u >> 20);
+        }
+        return r | (uint8_t)(sign >> 24);
+    }
+};
+template <> struct Elem<kF8E5M2> {
+    typedef uint8_t type;
+    static __device__ __forceinline__ uint8_t from_f32(float f) {
+        uint32_t u = f32_bits(f);
+        const uint32_t sign = u & 0x80000000u;
+        u ^= sign;
+        uint8_t r;
+        if (u >= (143u << 23)) {
+            r = u > (255u << 23) ? 0x7f : 0x7c; // NaN : infinity (65536 and above overflow)
+        } else if (u < (113u << 23)) {
+            const uint32_t magic = 134u << 23;
+            r = (uint8_t)(f32_bits(bits_f32(u) + bits_f32(magic)) - magic);
+        } else {
+            const uint32_t odd = (u >> 21) & 1u;
+            u += ((uint32_t)(15 - 127) << 23) + 0xfffffu + odd;
+            r = (uint8_t)(u >> 21);
+        }
+        return r | (uint8_t)(sign >> 24);
+    }
+};
+
+// a 16-byte vector that is only aligned like one element of N bytes
+template <int N> struct LooseVec;
+template <> struct LooseVec<2> { typedef v4u type __attribute__((aligned(2))); };
+template <> struct LooseVec<4> { typedef v4u type __attribute__((aligned(4))); };
+template <> struct LooseVec<8> { typedef v4u type __attribute__((aligned(8))); };
+
+template <int N> struct WordOf;
+template <> struct WordOf<2> { typedef uint16_t type; };
+template <> struct WordOf<4> { typedef uint32_t type; };
+template <> struct WordOf<8> { typedef uint64_t type; };
+template <> struct WordOf<16> { typedef v4u type; };
+
+// One 16-byte load per lane (16 / sizeof(src) elements), one narrower store per lane.
+template <uint32_t S, uint32_t D>
+__device__ __forceinline__ void convert_span(const ConvertJob &job, uint32_t lb) {
+    typedef typename Elem<S>::type src_t;
+    typedef typename Elem<D>::type dst_t;
+    constexpr uint32_t kPer = 16 / sizeof(src_t); // elements per lane
+    typedef typename WordOf<kPer * sizeof(dst_t)>::type out_t;
+    // the 16-byte load is only as aligned as one element: global loads of any width take
+    // element-aligned addresses on this hardware
+    typedef typename LooseVec<sizeof(src_t)>::type in_t;
+    const src_t *src = reinterpret_cast<const src_t *>(job.src);
+    dst_t *dst = reinterpret_cast<dst_t *>(job.dst);
+    const uint64_t first = ((uint64_t)lb * kBlock + threadIdx.x) * kPer;
+    if (first >= job.n_elems) return;
+    // the store needs its natural alignment
+    const bool wide = ((uintptr_t)job.dst & (sizeof(out_t) - 1)) == 0 && first + kPer <= job.n_elems;
+    if (wide) {
+        const v4u raw = *(const FSTX_GLOBAL in_t *)(src + first);
+        src_t in[kPer];
+        dst_t out[kPer];
+        __builtin_memcpy(in, &raw, 16);
+#pragma unroll
+        for (uint32_t k = 0; k < kPer; ++k) out[k] = Elem<D>::from_f32(Elem<S>::to_f32(in[k]));
+        out_t packed;
+        __builtin_memcpy(&packed, out, sizeof packed);
+        st_global(packed, reinterpret_cast<out_t *>(dst + first));
+    } else { // misaligned destination or the ragged end: element by element
+        for (uint32_t k = 0; k < kPer && first + k < job.n_elems; ++k)
+            st_global(Elem<D>::from_f32(Elem<S>::to_f32(ld_global(src + first + k))), dst + first + k);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t granule_log2,
+                                                          const JobTable<ConvertJob> t) {
+    const uint32_t b = blockIdx.x;
+    const uint32_t ji = find_job(t, granule_log2, b);
+    const ConvertJob job = t.fetch(ji);
+    const uint32_t lb = b - t.first_block[ji];
+#define FSTX_CONVERT(S, D) \
+    case (S) * 8 + (D): convert_span<S, D>(job, lb); break;
+    switch (job.src_type * 8 + job.dst_type) { // uniform across the workgroup
+        FSTX_CONVERT(kF64, kF32) FSTX_CONVERT(kF64, kF16) FSTX_CONVERT(kF64, kBF16)
+        FSTX_CONVERT(kF64, kF8E4M3) FSTX_CONVERT(kF64, kF8E5M2)
+        FSTX_CONVERT(kF32, kF16) FSTX_CONVERT(kF32, kBF16) FSTX_CONVERT(kF32, kF8E4M3) FSTX_CONVERT(kF32, kF8E5M2)
+        FSTX_CONVERT(kF16, kBF16) FSTX_CONVERT(kF16, kF8E4M3) FSTX_CONVERT(kF16, kF8E5M2)
+        FSTX_CONVERT(kBF16, kF16) FSTX_CONVERT(kBF16, kF8E4M3) FSTX_CONVERT(kBF16, kF8E5M2)
+    default: break; // rejected on the host
+    }
+#undef FSTX_CONVERT
 }
 
 // --------------------------------------------------------------- host side
@@ -520,4 +689,39 @@ extern "C" int fstx_slice_copy(void *dst, const void *src, uint64_t outer, uint6
                                uint64_t src_pitch, void *stream) {
     fstx_slice_desc d{dst, src, outer, seg_bytes, src_pitch};
     return fstx_slice_copy_batch(&d, 1, stream);
+}
+
+extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {
+    if (n == 0) return 0;
+    if (!descs) return -FSTX_E_INVAL;
+    if (n > FSTX_BATCH_MAX) return -FSTX_E_TOO_MANY;
+    static const uint32_t size_of[6] = {8, 4, 2, 2, 1, 1};
+    JobTable<ConvertJob> t;
+    uint64_t blocks_of[FSTX_BATCH_MAX];
+    uint64_t sum = 0;
+    uint32_t k = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const fstx_convert_desc &d = descs[i];
+        if (d.n_elems == 0) continue;
+        if (!d.dst || !d.src || d.src_type > FSTX_F8_E5M2 || d.dst_type > FSTX_F8_E5M2) return -FSTX_E_INVAL;
+        const uint32_t ss = size_of[d.src_type], ds = size_of[d.dst_type];
+        // only towards a type that is not wider, never from fp8, never onto the same type
+        if (ds > ss || d.src_type >= FSTX_F8_E4M3 || d.src_type == d.dst_type || d.dst_type == FSTX_F64) return -FSTX_E_INVAL;
+        if (((uintptr_t)d.src % ss) || ((uintptr_t)d.dst % ds)) return -FSTX_E_INVAL;
+        const char *sb = static_cast<const char *>(d.src);
+        char *db = static_cast<char *>(d.dst);
+        if (sb < db + d.n_elems * ds && db < sb + d.n_elems * ss) return -FSTX_E_INVAL; // overlap
+        t.job[k] = ConvertJob{db, sb, d.n_elems, d.src_type, d.dst_type};
+        const uint64_t per_block = (uint64_t)kBlock * (16 / ss);
+        blocks_of[k] = (d.n_elems + per_block - 1) / per_block;
+        sum += blocks_of[k];
+        if (sum > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
+        ++k;
+    }
+    if (k == 0) return 0;
+    uint32_t gl = 0;
+    const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
+    hipLaunchKernelGGL(convert_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                       gl, t);
+    return fstx_internal::check_launch("convert_kernel");
 }

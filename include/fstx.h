@@ -198,6 +198,31 @@ typedef struct fstx_slice_desc {
  * file_buffer.py:238-259). */
 int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, void *stream);
 
+/* element types of fstx_convert_batch */
+enum fstx_elem_type {
+    FSTX_F64 = 0,
+    FSTX_F32 = 1,
+    FSTX_F16 = 2,
+    FSTX_BF16 = 3,
+    FSTX_F8_E4M3 = 4, /* e4m3fn: no infinity, 0x7f / 0xff are NaN */
+    FSTX_F8_E5M2 = 5
+};
+
+typedef struct fstx_convert_desc {
+    void *dst;
+    const void *src;
+    uint64_t n_elems;
+    uint32_t src_type; /* enum fstx_elem_type */
+    uint32_t dst_type;
+} fstx_convert_desc;
+
+/* n <= FSTX_BATCH_MAX element-type conversions in one launch, out of place, towards a
+ * type that is not wider (f64 -> f32/f16/bf16/fp8, f32 -> f16/bf16/fp8, f16 <-> bf16,
+ * f16/bf16 -> fp8), with the rounding of torch's Tensor.to().  Replaces the per-tensor
+ * t2.to(dtype) + copy_ of SafeTensorsMetadata.get_tensors when copy_files_to_device is
+ * given a dtype (common.py:355-375). */
+int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
