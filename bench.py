@@ -46,7 +46,7 @@ HBM_PEAK_GBPS = 8000.0
 # according to rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by its reading for an aligned
 # 1 GiB copy (x1.99988 and x0.99965): profiles/fstx_kernels_hbm_traffic_counters.md.  Algorithmic:
 # 1,357,905,920.
-SLICE_KERNEL_TRAFFIC_BYTES = 1_357_731_888
+SLICE_KERNEL_TRAFFIC_BYTES = 1_357_747_660
 
 
 def log(*a):
@@ -211,7 +211,11 @@ def run_load(files: List[str], read_mode: str, threads: int, block_kb: int, veri
     metrics = loader.copier_constructor.reader.metrics()
     out = {"init_s": t1 - t0, "io_s": t2 - t1, "get_s": t3 - t2, "elapsed_s": t3 - t0, "bytes": nbytes,
            "blocks_direct": int(metrics.blocks_direct), "blocks_buffered": int(metrics.blocks_buffered),
-           "direct_depth": int(metrics.direct_depth)}
+           "direct_depth": int(metrics.direct_depth),
+           # summed over the I/O workers; with one O_DIRECT read in flight at a time,
+           # pread_s / io_s is the share of the load during which the disk was busy
+           "pread_s": metrics.read_ns / 1e9, "stage_memcpy_s": metrics.stage_ns / 1e9,
+           "slot_wait_s": metrics.slot_wait_ns / 1e9}
     if verify is not None:
         bad = [k for k, t in tensors.items() if checksum(t) != verify[k]]
         if bad:
@@ -270,6 +274,83 @@ def bench_tp_extract(files: List[str], world: int, threads: int, block_kb: int) 
                         f"columns of o/down, copies of the rest)",
             "seconds_per_rank": secs, "algorithmic_bytes": moved, "GBps": moved / 1e9 / total,
             "tensors_reassembled_and_compared": checked}
+
+
+def bench_multi_cols(files: List[str], world: int, threads: int, block_kb: int) -> dict:
+    """``get_multi_cols`` (fused slice + join: QKV and gate/up packing) for every layer and
+    every rank of a TP=``world`` stub group over the HBM-resident checkpoint.  Checked
+    against torch's slicing + cat of the whole tensors."""
+    import torch
+
+    from fastsafetensors_amd import SafeTensorsFileLoader, SingleGroup, StubProcessGroup
+
+    whole_loader = SafeTensorsFileLoader(SingleGroup(), "cuda:0", max_threads=threads, block_size_kb=block_kb)
+    whole_loader.add_filenames({0: files})
+    whole = whole_loader.copy_files_to_device()
+    layers = sorted({int(k.split(".")[2]) for k in whole_loader.get_keys() if k.startswith("model.layers.")})
+    groups = []
+    for i in layers:
+        p = f"model.layers.{i}."
+        groups.append([p + f"self_attn.{x}_proj.weight" for x in "qkv"])
+        groups.append([p + f"mlp.{x}_proj.weight" for x in ("gate", "up")])
+    secs, moved, checked = [], 0, 0
+    for rank in range(world):
+        loader = SafeTensorsFileLoader(StubProcessGroup(rank, world), "cuda:0", max_threads=threads,
+                                       block_size_kb=block_kb)
+        loader.add_filenames({rank: files})
+        bufs = loader.copy_files_to_device()
+        bufs.auto_mem_delete = False
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = [bufs.get_multi_cols(names, dim=0) for names in groups]
+        torch.cuda.synchronize()
+        secs.append(time.perf_counter() - t0)
+        moved += sum(2 * t.get_raw().numel() * t.get_raw().element_size() for t in outs)
+        for names, t in list(zip(groups, outs))[:: max(1, len(groups) // 8)]:
+            parts = []
+            for n in names:
+                full = whole.get_tensor(n)
+                block = -(-full.shape[0] // world)
+                parts.append(full[rank * block : (rank + 1) * block])
+            if not torch.equal(t.get_raw(), torch.cat(parts, dim=0)):
+                raise SystemExit(f"bench: get_multi_cols({names}) differs from slicing + cat")
+            checked += 1
+        del outs
+        bufs.close()
+        loader.close()
+    whole.close()
+    whole_loader.close()
+    return {"workload": f"get_multi_cols of [q,k,v] and [gate,up] (dim 0) for {len(layers)} layers, each of {world} ranks",
+            "calls_per_rank": len(groups), "seconds_per_rank": secs, "algorithmic_bytes": moved,
+            "GBps": moved / 1e9 / sum(secs), "joined_tensors_compared": checked}
+
+
+def bench_iterate_weights(files: List[str], threads: int, verify) -> dict:
+    """``ParallelLoader.iterate_weights`` over the checkpoint, warm page cache: the next file
+    loads while the tensors of the current one are copied out and handed to the caller."""
+    import torch
+
+    from fastsafetensors_amd import ParallelLoader
+
+    out = {}
+    for check in (False, True):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        it = ParallelLoader(None, files, device="cuda:0", max_threads=threads)
+        nbytes = count = 0
+        for name, t in it.iterate_weights():
+            nbytes += t.numel() * t.element_size()
+            count += 1
+            if check and checksum(t) != verify[name]:
+                raise SystemExit(f"bench: iterate_weights handed out wrong bytes for {name}")
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        it.close()
+        if not check:
+            out = {"workload": "ParallelLoader.iterate_weights, queue_size=0, every tensor copied out of its file buffer",
+                   "tensors": count, "bytes": nbytes, "seconds": dt, "GBps": nbytes / 1e9 / dt}
+    out["tensors_checksum_verified"] = count
+    return out
 
 
 # ---- kernels ------------------------------------------------------------------------------------------
@@ -404,7 +485,7 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     }
     # -- down-cast on load: fp32 -> bf16 over 1 GiB of fp32 in 48 tensors per launch
     #    (4 bytes read + 2 written per element)
-    per = cal // 4 // 48 // 16 * 16
+    per = cal // 4 // 48 // 64 * 64  # whole 256-byte spans, so that no cache line is shared between two jobs
     src32 = window[: cal].view(torch.float32)
     dst16 = dst[: cal // 2].view(torch.int16)
     cjobs = [(dst16.data_ptr() + 2 * i * per, src32.data_ptr() + 4 * i * per, per,
@@ -426,6 +507,46 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         "launches_timed": len(times), "avg_launch_ms": avg_ms, "bytes_per_launch": 2 * n,
         "achieved_GBps": 2 * n / 1e6 / avg_ms, "best_GBps": 2 * n / 1e6 / min(times),
     }
+    return out
+
+
+def bench_downcast(data_dir: str, threads: int) -> dict:
+    """GPT-2-small fp32 (config C1, 497,759,232 data bytes) loaded warm as stored and with a
+    down-cast to fp16 / bf16 on load -- the case of the reference's published figure
+    (docs/amd-perf.md:73,77: 2.07 GB/s as stored, 0.77 GB/s with the F16 cast, MI300X)."""
+    import torch
+
+    from fastsafetensors_amd import DType, SafeTensorsFileLoader, SingleGroup
+    from fastsafetensors_amd import checkpoints as ck
+
+    recs = ck.write_config(ck.configs(1.0)["C1"], data_dir, device="cuda", sha256=False)
+    path = recs[0]["path"]
+    nbytes = recs[0]["size"] - recs[0]["header_length"]
+    warm_cache([path])
+    out = {"workload": f"C1 GPT-2-small fp32, {nbytes} data bytes, warm page cache; GB/s counts the file's bytes"}
+    ref = None
+    for label, dtype, tdt in [("as_stored", DType.AUTO, None), ("to_f16", DType.F16, torch.float16),
+                              ("to_bf16", DType.BF16, torch.bfloat16)]:
+        best = None
+        for rep in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            loader = SafeTensorsFileLoader(SingleGroup(), "cuda:0", max_threads=threads)
+            loader.add_filenames({0: [path]})
+            bufs = loader.copy_files_to_device(dtype=dtype)
+            tensors = {k: bufs.get_tensor(k) for k in loader.get_keys()}
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            if rep == 0:
+                if ref is None:
+                    ref = {k: t.clone() for k, t in tensors.items()}
+                elif not all(torch.equal(t.view(torch.int16), ref[k].to(tdt).view(torch.int16)) for k, t in tensors.items()):
+                    raise SystemExit(f"bench: tensors loaded with dtype={dtype} differ from Tensor.to()")
+            del tensors
+            bufs.close()
+            loader.close()
+        out[label] = {"seconds_best_of_3": best, "GBps": nbytes / 1e9 / best}
     return out
 
 
@@ -562,37 +683,40 @@ def main() -> None:
         log(f"[bench] ceilings: pinned H2D {h2d:.2f} GB/s, page cache read {pagecache:.1f} GB/s "
             f"(resident after drop {cold_frac:.3f}, after warm-up {warm_frac:.3f})")
 
-        probe_at = [0]
-        total_size = sum(os.path.getsize(f) for f in files)
+        probe_no = [0]
 
         def raw_disk_rate() -> float:
-            """What the disk delivers right now to a plain sequential O_DIRECT reader
-            (best of two request sizes, 1 GiB each, a fresh region every call)."""
-            best = 0.0
-            for th, blk in [(1, 16 << 20), (1, 64 << 20)]:
-                nb, dt = parallel_read(files, direct=True, threads=th, limit=1 << 30, block=blk, start=probe_at[0])
-                probe_at[0] = (probe_at[0] + (1 << 30)) % max(1, total_size - (2 << 30))
-                best = max(best, nb / 1e9 / dt)
-            return best
+            """What the disk delivers right now to a plain sequential O_DIRECT reader that
+            reads the same bytes as a load does: the whole checkpoint, cold, 64 MiB requests,
+            two readers and one reader on alternate calls.  (Short probes catch the
+            burst rate of this throttled virtual disk, 6-8 GB/s for 1 GiB, which no reader
+            sustains over 16 GB.)"""
+            readers = (2, 1)[probe_no[0] % 2]
+            probe_no[0] += 1
+            drop_cache(files)
+            nb, dt = parallel_read(files, direct=True, threads=readers, limit=None, block=64 << 20)
+            return nb / 1e9 / dt
 
         def steps_of(kind: str, n: int, check: bool) -> List[Dict[str, float]]:
             runs = []
             for i in range(n):
                 before = None
                 if kind == "cold":
+                    before = last_raw[0] if last_raw[0] is not None else raw_disk_rate()
                     drop_cache(files)
-                    before = raw_disk_rate()
                 r = run_load(files, "auto", args.threads, args.block_kb, verify if (check and i == 0) else None)
                 if kind == "cold":
                     # the disk is shared and throttled in bursts: its ceiling is taken right
                     # around the step, not once at the start
-                    r["disk_GBps_around_step"] = [before, raw_disk_rate()]
+                    last_raw[0] = raw_disk_rate()
+                    r["disk_GBps_around_step"] = [before, last_raw[0]]
                 runs.append(r)
                 log(f"[bench] {kind} step {i}: elapsed {r['elapsed_s']:.3f}s io {r['io_s']:.3f}s "
-                    f"-> {r['bytes'] / 1e9 / r['elapsed_s']:.2f} GB/s (direct blocks {r['blocks_direct']}, buffered {r['blocks_buffered']}"
+                    f"-> {r['bytes'] / 1e9 / r['elapsed_s']:.2f} GB/s (direct blocks {r['blocks_direct']}, buffered {r['blocks_buffered']}, in pread {r['pread_s']:.2f}s, staging memcpy {r['stage_memcpy_s']:.2f}s, slot wait {r['slot_wait_s']:.2f}s"
                     + (f", raw O_DIRECT reader before/after {r['disk_GBps_around_step'][0]:.2f}/{r['disk_GBps_around_step'][1]:.2f} GB/s)" if kind == "cold" else ")"))
             return runs
 
+        last_raw = [None]  # a whole-checkpoint raw read sits between every two cold loads
         steps_of("cold", args.warmup, False)
         cold = steps_of("cold", args.steps, True)
         drop_cache(files)
@@ -606,11 +730,18 @@ def main() -> None:
 
         tp = bench_tp_extract(files, 4, args.threads, args.block_kb)
         log(f"[bench] TP=4 as_dict over the resident checkpoint: {tp['GBps']:.0f} GB/s, seconds per rank {[round(x, 4) for x in tp['seconds_per_rank']]}")
+        mc = bench_multi_cols(files, 4, args.threads, args.block_kb)
+        log(f"[bench] TP=4 get_multi_cols (QKV, gate/up) over the resident checkpoint: {mc['GBps']:.0f} GB/s, seconds per rank {[round(x, 4) for x in mc['seconds_per_rank']]}")
+        itw = bench_iterate_weights(files, args.threads, verify)
+        log(f"[bench] iterate_weights warm: {itw['GBps']:.1f} GB/s ({itw['seconds']:.3f} s)")
+        downcast = bench_downcast(os.path.join(args.dir, "C1_downcast"), args.threads)
+        log(f"[bench] C1 fp32 warm load: " + ", ".join(f"{k} {v['GBps']:.1f} GB/s" for k, v in downcast.items() if isinstance(v, dict)))
         kernels = {} if args.skip_kernels else bench_kernels(args.steps, args.warmup)
         base = None if args.skip_cpu_baseline else cpu_baseline(files)
     finally:
         if not args.keep:
             shutil.rmtree(data_dir, ignore_errors=True)
+        shutil.rmtree(os.path.join(args.dir, "C1_downcast"), ignore_errors=True)
 
     def summarize(runs, ceiling):
         el = sorted(r["elapsed_s"] for r in runs)
@@ -620,13 +751,14 @@ def main() -> None:
                 "io_GBps_median": data_bytes / 1e9 / sorted(r["io_s"] for r in runs)[len(runs) // 2],
                 "roofline_GBps": ceiling, "frac_of_roofline": gbps / ceiling}
 
-    local = sorted(sum(r["disk_GBps_around_step"]) / 2 for r in cold)
+    local = sorted(max(r["disk_GBps_around_step"]) for r in cold)
     disk_local = local[len(local) // 2]
     cold_s = summarize(cold, min(disk_local, h2d))
-    fr = sorted(r["bytes"] / 1e9 / r["elapsed_s"] / min(sum(r["disk_GBps_around_step"]) / 2, h2d) for r in cold)
+    fr = sorted(r["bytes"] / 1e9 / r["elapsed_s"] / min(max(r["disk_GBps_around_step"]), h2d) for r in cold)
     cold_s["frac_of_roofline_per_step_median"] = fr[len(fr) // 2]
-    cold_s["roofline_note"] = ("roofline = min(raw sequential O_DIRECT read rate measured right before and after each cold step, "
-                               "pinned H2D); the disk is a throttled shared virtual disk whose rate drifts by 2-3x within a run")
+    cold_s["roofline_note"] = ("roofline = min(rate of a plain sequential O_DIRECT reader over the same whole checkpoint, the faster of "
+                               "the runs right before and right after each cold step, pinned H2D); the disk is a throttled shared virtual disk whose "
+                               "rate drifts within a run and bursts for short reads")
     warm_s = summarize(warm, min(pagecache, h2d))
     line = {
         "metric": "file->HBM GB/s, cold page cache, Llama-3-8B bf16 checkpoint (whole load: ctor to last tensor)",
@@ -653,6 +785,9 @@ def main() -> None:
                      "parity": f"{cold[0].get('verified_tensors', 0)} tensors checksum-verified on the GPU after a cold and a warm load"},
     }
     line["tp_extract"] = tp
+    line["multi_cols"] = mc
+    line["iterate_weights"] = itw
+    line["downcast_on_load"] = downcast
     if kernels:
         k = kernels["slice_extract"]
         line["roofline"] = {"bound": "hbm", "achieved": k["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
