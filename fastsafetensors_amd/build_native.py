@@ -4,8 +4,8 @@
     python -m fastsafetensors_amd.build_native
 
 hipcc cross-compiles without a GPU.  ``-packed-fp32-ops`` is switched off for
-device code on purpose (the kernels contain no float arithmetic, the flag keeps
-it that way for anything added later).
+device code on purpose: the conversion kernel's float arithmetic must not be
+compiled into packed FP32 instructions.
 """
 import os
 import shutil

@@ -245,20 +245,30 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
 // For segments whose length, pitch or source address is not a multiple of 16
 // bytes the direct kernel above has to drop to 8-, 4-, 2- or 1-byte moves per
 // lane.  This variant keeps every global access 16 bytes wide: a wavefront owns
-// a 4 KiB tile of the (16-byte aligned) destination, loads the aligned 16-byte
+// a 2 KiB tile of the (16-byte aligned) destination, loads the aligned 16-byte
 // source vectors that cover the tile's rows into LDS -- each row into its own
-// slot, at the same offset modulo 16 it has in memory -- and then assembles each
-// destination vector from naturally aligned `unit`-sized LDS reads.  The odd
-// alignment is absorbed by LDS, whose banks do not care about it.
+// slot, at the same offset modulo 16 it has in memory -- and then reads each
+// destination vector back with one 16-byte LDS read at the byte address where its
+// data begins.  The odd alignment is absorbed by LDS, which serves unaligned reads.
 
-constexpr uint32_t kTileBytes = 4096; // destination bytes per wavefront
+#ifndef FSTX_LDS_TILE
+#define FSTX_LDS_TILE 2048
+#endif
+constexpr uint32_t kTileBytes = FSTX_LDS_TILE; // destination bytes per wavefront
 constexpr uint32_t kLdsMinSeg = 64;   // shorter segments stay on the direct kernel
 // LDS slot of the tile's i-th row piece starts at align_down(s_i + 48 i, 16), where s_i is
 // the piece's position in the tile: consecutive slots then never overlap (a piece of L bytes
 // needs at most L + 30 bytes once both ends are widened to 16-byte vectors), and a tile
-// touches at most floor(4094 / 64) + 2 = 65 rows.
+// touches at most floor((tile - 2) / seg) + 2 rows.
 constexpr uint32_t kRowGap = 48;
-constexpr uint32_t kLdsBytes = kTileBytes + kRowGap * 66 + 64;
+// LDS a wavefront needs when no segment of the launch is shorter than min_seg: the fewer rows
+// a tile can touch, the less LDS per wavefront and the more wavefronts a CU keeps in flight
+// (3.7 KB at 64-byte segments, 2.3 KB from 2 KiB segments up).  2 KiB tiles measured a
+// little faster than 4 KiB ones (5.5 against 5.3 TB/s), 1 KiB and 8 KiB ones slower.
+inline uint32_t lds_bytes_for(uint64_t min_seg) {
+    const uint32_t rows = (uint32_t)((kTileBytes - 2) / min_seg) + 2;
+    return kTileBytes + kRowGap * (rows + 1) + 64;
+}
 
 struct alignas(32) LdsSliceJob {
     char *dst;            // 16-byte aligned
@@ -268,117 +278,126 @@ struct alignas(32) LdsSliceJob {
     uint32_t outer;       // number of segments
 };
 
-template <int U> struct UnitOf;
-template <> struct UnitOf<1> { typedef uint8_t type; };
-template <> struct UnitOf<2> { typedef uint16_t type; };
-template <> struct UnitOf<4> { typedef uint32_t type; };
-template <> struct UnitOf<8> { typedef uint64_t type; };
-
-// geometry of one tile: which rows it touches and where each row piece sits
+// Geometry of one tile in 32-bit arithmetic.  Positions are counted in bytes from column 0
+// of the tile's first row: destination byte p of the tile is position first_col + p, local
+// row i covers positions [i * seg, (i + 1) * seg).  seg < 2^31 keeps all of it below 2^32.
 struct TileGeom {
-    const char *src;
-    uint64_t pitch, d0, d1, row_first, row_last;
-    uint32_t seg, first_col;
+    uint32_t seg, first_col, end_pos, src_lo, pitch_lo;
 
-    __device__ __forceinline__ uint32_t col_begin(uint64_t row) const { return row == row_first ? first_col : 0; }
-    __device__ __forceinline__ uint32_t col_end(uint64_t row) const {
-        return row == row_last ? (uint32_t)(d1 - row_last * seg) : seg;
-    }
-    __device__ __forceinline__ uintptr_t src_begin(uint64_t row) const {
-        return (uintptr_t)src + row * pitch + col_begin(row);
-    }
-    // LDS offset of the 16-byte vector that holds the row piece's first source byte
-    __device__ __forceinline__ uint32_t slot(uint64_t row) const {
-        const uint32_t i = (uint32_t)(row - row_first);
-        const uint32_t s = i == 0 ? 0u : (uint32_t)(row * seg - d0);
+    __device__ __forceinline__ uint32_t col_begin(uint32_t i) const { return i == 0 ? first_col : 0u; }
+    // LDS offset of the 16-byte vector that receives the first source vector of row piece i
+    __device__ __forceinline__ uint32_t slot(uint32_t i) const {
+        const uint32_t s = i * seg + col_begin(i) - first_col; // where the piece starts in the tile
         return (s + kRowGap * i) & ~15u;
+    }
+    // LDS offset of column 0 of local row i (for row 0 it may lie before the slot; the
+    // difference wraps consistently in 32 bits and is only used with col >= col_begin)
+    __device__ __forceinline__ uint32_t row_base(uint32_t i) const {
+        const uint32_t cb = col_begin(i);
+        const uint32_t mis = (src_lo + i * pitch_lo + cb) & 15u; // the piece's source address mod 16
+        return slot(i) + mis - cb;
     }
 };
 
-template <int U>
-__device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, unsigned char *lds) {
-    typedef typename UnitOf<U>::type unit_t;
-    const uint32_t lane = threadIdx.x;
-    TileGeom g;
-    g.src = job.src;
-    g.pitch = job.pitch_unit & 0x00ffffffffffffffull;
-    g.seg = job.seg_bytes;
-    const uint64_t total = (uint64_t)job.outer * g.seg;
-    g.d0 = (uint64_t)tile * kTileBytes;
-    g.d1 = g.d0 + kTileBytes < total ? g.d0 + kTileBytes : total;
-    g.row_first = g.d0 / g.seg;
-    g.row_last = (g.d1 - 1) / g.seg;
-    g.first_col = (uint32_t)(g.d0 - g.row_first * g.seg);
-    const uint32_t nrows = (uint32_t)(g.row_last - g.row_first) + 1;
+// 16 bytes of LDS at any byte address (the hardware runs DS operations in unaligned mode)
+typedef v4u lds_vec __attribute__((aligned(1)));
 
-    // ---- phase 1: aligned 16-byte loads.  `group` lanes share a row piece; short rows are
-    // loaded several per step so that the lanes stay busy.
-    const uint32_t longest = g.seg < kTileBytes ? g.seg : kTileBytes;
+__device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, unsigned char *lds) {
+    const uint32_t lane = threadIdx.x;
+    const uint64_t pitch = job.pitch_unit & 0x00ffffffffffffffull;
+    const uint32_t seg = job.seg_bytes;
+    const uint64_t total = (uint64_t)job.outer * seg;
+    const uint64_t d0 = (uint64_t)tile * kTileBytes;
+    const uint32_t tile_bytes = total - d0 < kTileBytes ? (uint32_t)(total - d0) : kTileBytes;
+    // the tile's first row; a 32-bit division whenever the job is smaller than 4 GiB
+    const uint64_t row_first = (total >> 32) == 0 ? (uint64_t)((uint32_t)d0 / seg) : d0 / seg;
+    TileGeom g;
+    g.seg = seg;
+    g.first_col = (uint32_t)(d0 - row_first * seg);
+    g.end_pos = g.first_col + tile_bytes;
+    g.pitch_lo = (uint32_t)pitch;
+    g.src_lo = (uint32_t)(uintptr_t)job.src + (uint32_t)row_first * g.pitch_lo; // low address bits are all that matter
+    const uint32_t nrows = (g.end_pos - 1) / seg + 1;
+    const char *src_row0 = job.src + row_first * pitch;
+
+    // ---- phase 1: aligned 16-byte loads into LDS.  `group` lanes share a row piece; short
+    // rows are loaded several per step so that the lanes stay busy.
+    const uint32_t longest = seg < kTileBytes ? seg : kTileBytes;
     const uint32_t vmax = (longest + 30) / 16 + 1; // vectors a row piece can need
-    uint32_t group = 64;
-    while (group / 2 >= vmax) group /= 2;
-    const uint32_t rows_per_step = 64 / group;
-    for (uint32_t ibase = 0; ibase < nrows; ibase += rows_per_step) {
-        const uint32_t i = ibase + lane / group;
+    uint32_t group_log2 = 6;
+    while (group_log2 > 0 && (32u >> (6 - group_log2)) >= vmax) --group_log2;
+    const uint32_t group = 1u << group_log2;
+    for (uint32_t ibase = 0; ibase < nrows; ibase += 64u >> group_log2) {
+        const uint32_t i = ibase + (lane >> group_log2);
         if (i < nrows) {
-            const uint64_t row = g.row_first + i;
-            const uintptr_t a0 = g.src_begin(row), a1 = a0 + (g.col_end(row) - g.col_begin(row));
+            const uint32_t cb = g.col_begin(i);
+            const uint32_t pos_end = (i + 1) * seg < g.end_pos ? (i + 1) * seg : g.end_pos;
+            const uintptr_t a0 = (uintptr_t)src_row0 + (uint64_t)i * pitch + cb;
+            const uintptr_t a1 = a0 + (pos_end - (i * seg + cb));
             const uintptr_t lo = a0 & ~(uintptr_t)15;
-            const uint32_t at = g.slot(row);
-            for (uint32_t v = lane % group; lo + 16ull * v < a1; v += group)
+            const uint32_t at = g.slot(i);
+            for (uint32_t v = lane & (group - 1); lo + 16ull * v < a1; v += group)
                 *reinterpret_cast<v4u *>(lds + at + 16 * v) = ld_stream(reinterpret_cast<const v4u *>(lo) + v);
         }
     }
     __syncthreads(); // one wavefront: orders its LDS writes before the reads below
 
-    // ---- phase 2: every lane assembles its destination vectors from LDS
-    for (uint64_t d = g.d0 + 16ull * lane; d < g.d1; d += 16 * 64) {
-        uint64_t row = d / g.seg;
-        uint32_t col = (uint32_t)(d - row * g.seg);
-        // LDS address of column `col` of `row` = bias + col
-        auto bias_of = [&](uint64_t r) -> int32_t {
-            return (int32_t)(g.slot(r) + ((uint32_t)g.src_begin(r) & 15u)) - (int32_t)g.col_begin(r);
-        };
-        int32_t bias = bias_of(row);
-        const uint32_t nbytes = g.d1 - d < 16 ? (uint32_t)(g.d1 - d) : 16u;
-        unit_t piece[16 / U];
+    // ---- phase 2: one 16-byte LDS read per destination vector, at whatever alignment the
+    // source had; a vector that runs over the end of a row takes its remaining bytes from
+    // the start of the next row (rows are at least 64 bytes, so never from a third).
+    for (uint32_t p = 16 * lane; p < tile_bytes; p += 16 * 64) {
+        const uint32_t pos = g.first_col + p;
+        const uint32_t i = pos / seg;
+        const uint32_t col = pos - i * seg;
+        const uint32_t n = tile_bytes - p < 16 ? tile_bytes - p : 16u; // < 16 only at the end of the job
+        const uint32_t in_row = seg - col;
+        v4u out = *reinterpret_cast<const lds_vec *>(lds + (g.row_base(i) + col));
+        if (in_row < n) {
+            const v4u next = *reinterpret_cast<const lds_vec *>(lds + (g.row_base(i + 1) - in_row));
+            uint32_t o[4] = {out.x, out.y, out.z, out.w};
+            const uint32_t x[4] = {next.x, next.y, next.z, next.w};
 #pragma unroll
-        for (int p = 0; p < 16 / U; ++p) {
-            piece[p] = 0;
-            if ((uint32_t)p * U < nbytes) {
-                piece[p] = *reinterpret_cast<const unit_t *>(lds + (bias + (int32_t)col));
-                col += U;
-                if (col >= g.seg) {
-                    col = 0;
-                    ++row;
-                    if (row <= g.row_last) bias = bias_of(row);
-                }
+            for (int w = 0; w < 4; ++w) {
+                // bytes of this dword that still belong to the current row: 0..4
+                const int keep = (int)in_row - 4 * w;
+                const uint32_t m = keep >= 4 ? 0xffffffffu : keep <= 0 ? 0u : (1u << (8 * keep)) - 1u;
+                o[w] = (o[w] & m) | (x[w] & ~m);
             }
+            out = v4u{o[0], o[1], o[2], o[3]};
         }
-        if (nbytes == 16) {
-            v4u out;
-            __builtin_memcpy(&out, piece, 16);
-            st_stream(out, reinterpret_cast<v4u *>(job.dst + d));
+        char *dst = job.dst + d0 + p;
+        if (n == 16) {
+            st_stream(out, reinterpret_cast<v4u *>(dst));
         } else { // the job's last, partial vector
-            for (uint32_t p = 0; p * U < nbytes; ++p) st_global(piece[p], reinterpret_cast<unit_t *>(job.dst + d) + p);
+            const uint32_t o[4] = {out.x, out.y, out.z, out.w};
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+                if ((uint32_t)q < n) st_global((unsigned char)(o[q / 4] >> (8 * (q % 4))), reinterpret_cast<unsigned char *>(dst) + q);
         }
     }
 }
 
 __global__ __launch_bounds__(64) void slice_lds_kernel(const uint32_t granule_log2,
                                                        const JobTable<LdsSliceJob> t) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[kLdsBytes];
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[]; // lds_bytes_for(shortest segment)
     const uint32_t b = blockIdx.x;
     const uint32_t ji = find_job(t, granule_log2, b);
     const LdsSliceJob job = t.fetch(ji);
-    const uint32_t tile = b - t.first_block[ji];
-    if ((uint64_t)tile * kTileBytes >= (uint64_t)job.outer * job.seg_bytes) return; // idle granule padding
-    switch ((uint32_t)(job.pitch_unit >> 56)) { // uniform across the workgroup
-    case 3: lds_tile<8>(job, tile, lds); break;
-    case 2: lds_tile<4>(job, tile, lds); break;
-    case 1: lds_tile<2>(job, tile, lds); break;
-    default: lds_tile<1>(job, tile, lds); break;
-    }
+    const uint32_t lb = b - t.first_block[ji];
+    // Neighbouring tiles share the source cache lines that their common border cuts through.
+    // Workgroups go round-robin over the eight dies, so give each die one contiguous eighth of
+    // the job's tiles: the shared line is then found in that die's L2 instead of being fetched twice.
+    const uint64_t n_tiles = ((uint64_t)job.outer * job.seg_bytes + kTileBytes - 1) / kTileBytes;
+    const uint32_t per_die = (uint32_t)((n_tiles + kXcds - 1) / kXcds);
+#ifdef FSTX_LDS_NO_XCD_MAP
+    const uint32_t tile = lb;
+    if (tile >= n_tiles) return;
+#else
+    const uint32_t turn = lb / kXcds;
+    const uint32_t tile = (lb % kXcds) * per_die + turn;
+    if (turn >= per_die || tile >= n_tiles) return; // idle padding of the last eighth and granule
+#endif
+    lds_tile(job, tile, lds);
 }
 
 // ------------------------------------------------- down-cast while loading
@@ -607,16 +626,17 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     JobTable<SliceJob> t;
     JobTable<LdsSliceJob> tl;
     uint64_t blocks_of[FSTX_BATCH_MAX], tiles_of[FSTX_BATCH_MAX];
-    uint64_t blocks = 0, tiles = 0;
+    uint64_t blocks = 0, tiles = 0, min_seg = ~0ull;
     uint32_t k = 0, kl = 0;
     auto flush_lds = [&]() -> int {
         if (kl == 0) return 0;
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(tl, tiles_of, kl, &gl);
-        hipLaunchKernelGGL(slice_lds_kernel, dim3((uint32_t)grid), dim3(64), 0,
+        hipLaunchKernelGGL(slice_lds_kernel, dim3((uint32_t)grid), dim3(64), lds_bytes_for(min_seg),
                            static_cast<hipStream_t>(stream), gl, tl);
         kl = 0;
         tiles = 0;
+        min_seg = ~0ull;
         return fstx_internal::check_launch("slice_lds_kernel");
     };
     auto flush = [&]() -> int {
@@ -645,18 +665,19 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         uint64_t outer = d.outer, seg = d.seg_bytes, pitch = d.src_pitch;
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src |
                                              seg | pitch | 16u);
-        if (ul < 4 && seg >= kLdsMinSeg && seg <= 0xffffffffull && outer <= 0xffffffffull &&
+        if (ul < 4 && seg >= kLdsMinSeg && seg < 0x80000000ull && outer <= 0xffffffffull &&
             ((uintptr_t)d.dst & 15) == 0 && !fstx_internal::lds_path_disabled()) {
             // odd alignment somewhere: keep the global accesses 16 bytes wide and realign through LDS
             const uint64_t n_tiles = (outer * seg + kTileBytes - 1) / kTileBytes;
-            if (kl == FSTX_BATCH_MAX || tiles + n_tiles > kMaxBlocksPerLaunch) {
+            if (kl == FSTX_BATCH_MAX || tiles + n_tiles + kXcds > kMaxBlocksPerLaunch) {
                 int rc = flush_lds();
                 if (rc < 0) return rc;
             }
             tl.job[kl] = LdsSliceJob{static_cast<char *>(d.dst), static_cast<const char *>(d.src),
                                      pitch | ((uint64_t)ul << 56), (uint32_t)seg, (uint32_t)outer};
-            tiles_of[kl] = n_tiles;
-            tiles += n_tiles;
+            tiles_of[kl] = (n_tiles + kXcds - 1) / kXcds * kXcds; // whole eighths
+            tiles += tiles_of[kl];
+            if (seg < min_seg) min_seg = seg;
             ++kl;
             continue;
         }

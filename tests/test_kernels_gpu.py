@@ -225,6 +225,30 @@ def test_slice_odd_shapes_go_through_lds(dev):
                     assert (got[want.numel() :] == 77).all(), "wrote past the end of the shard"
 
 
+def test_slice_lds_random_geometry_in_one_batch(dev):
+    """Byte-level sweep of the LDS-staged kernel: segment lengths around the tile size and
+    its fractions, odd pitches, every source alignment, jobs of very different segment
+    lengths sharing one launch (the launch's LDS size follows the shortest segment)."""
+    rng = np.random.default_rng(23)
+    segs = [64, 65, 79, 81, 127, 129, 255, 511, 513, 1023, 1025, 2046, 2047, 2049, 2050, 4094, 4095, 4097, 6001, 8191]
+    for _ in range(6):
+        jobs, checks = [], []
+        for _j in range(24):
+            seg = int(rng.choice(segs))
+            pitch = seg + int(rng.choice([1, 2, 3, 7, 13, 16, 17, 100, 1001]))
+            outer = int(rng.integers(2, 40)) if seg < 3000 else int(rng.integers(2, 6))
+            shift = int(rng.integers(0, 16))
+            src = torch.randint(0, 255, (shift + outer * pitch + 32,), dtype=torch.uint8, device=dev)
+            dst = torch.full((outer * seg + 48,), 201, dtype=torch.uint8, device=dev)
+            jobs.append((dst.data_ptr(), src.data_ptr() + shift, outer, seg, pitch))
+            checks.append((src, dst, shift, outer, seg, pitch))
+        _native.slice_copy_batch(jobs, stream())
+        for src, dst, shift, outer, seg, pitch in checks:
+            want = src[shift : shift + outer * pitch].view(outer, pitch)[:, :seg].reshape(-1)
+            assert torch.equal(dst[: outer * seg], want), (seg, pitch, outer, shift)
+            assert (dst[outer * seg :] == 201).all(), "wrote past the end"
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
