@@ -442,8 +442,10 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     # -- slice extract on shapes whose rows are not multiples of 16 bytes: the LDS-staged
     #    kernel against the direct kernel at the small unit such shapes force
     odd = {}
-    for label, shape, tdt in [("bf16 [11008, 4090] cut in 4 along dim 1 (2046-byte segments, 8180-byte pitch)", (11008, 4090), torch.int16),
-                              ("fp8 [8192, 8190] cut in 4 along dim 1 (2048-byte segments, 8190-byte pitch)", (8192, 8190), torch.uint8),
+    # (inputs of 0.5 GB each: larger than the 256 MB memory-side cache, so that repeated launches
+    #  are served by HBM)
+    for label, shape, tdt in [("bf16 [65536, 4090] cut in 4 along dim 1 (2046-byte segments, 8180-byte pitch)", (65536, 4090), torch.int16),
+                              ("fp8 [65536, 8190] cut in 4 along dim 1 (2048-byte segments, 8190-byte pitch)", (65536, 8190), torch.uint8),
                               ("bf16 [32768, 8188] cut in 4 along dim 1 (4094-byte segments, 16376-byte pitch)", (32768, 8188), torch.int16)]:
         t = torch.randint(0, 100, shape, dtype=tdt, device=dev)
         item = t.element_size()
