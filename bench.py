@@ -690,14 +690,14 @@ def main() -> None:
 
         def raw_disk_rate() -> float:
             """What the disk delivers right now to a plain sequential O_DIRECT reader that
-            reads the same bytes as a load does: the whole checkpoint, cold, 64 MiB requests,
-            two readers and one reader on alternate calls.  (Short probes catch the
-            burst rate of this throttled virtual disk, 6-8 GB/s for 1 GiB, which no reader
-            sustains over 16 GB.)"""
-            readers = (2, 1)[probe_no[0] % 2]
+            reads the same bytes as a load does: the whole checkpoint, cold, one reader,
+            1 GiB and 256 MiB requests on alternate calls (the fastest plain patterns found
+            on this disk; more readers or smaller requests are slower).  Short probes catch
+            the burst rate of this throttled virtual disk, so every probe reads everything."""
+            blk = (1 << 30, 256 << 20)[probe_no[0] % 2]
             probe_no[0] += 1
             drop_cache(files)
-            nb, dt = parallel_read(files, direct=True, threads=readers, limit=None, block=64 << 20)
+            nb, dt = parallel_read(files, direct=True, threads=1, limit=None, block=blk)
             return nb / 1e9 / dt
 
         def steps_of(kind: str, n: int, check: bool) -> List[Dict[str, float]]:

@@ -147,6 +147,23 @@ struct Block {
     char *dev;         // device address of the first payload byte
 };
 
+// A staging buffer on loan: goes back to its context's pool when the last block that
+// still has bytes in it has been copied to the ring.
+struct StageLoan {
+    fstx_ctx *ctx;
+    char *stage;
+    StageLoan(fstx_ctx *c, char *s) : ctx(c), stage(s) {}
+    ~StageLoan();
+};
+
+// One block whose bytes an O_DIRECT read left in a staging buffer; any worker may
+// move it into the ring and on to the device.
+struct Staged {
+    Block block;
+    const char *bytes = nullptr;
+    std::shared_ptr<StageLoan> loan;
+};
+
 struct Slot {
     char *host = nullptr;
     fstx_dev::event_t ev = nullptr;
@@ -234,6 +251,7 @@ struct fstx_ctx {
     std::mutex q_mutex;
     std::condition_variable q_cv;
     std::deque<Block> queue;
+    std::deque<Staged> staged; // read by O_DIRECT, waiting for a worker to ship them (q_mutex)
     bool closing = false;
 
     std::mutex done_mutex;
@@ -256,6 +274,14 @@ struct fstx_ctx {
 };
 
 namespace {
+
+StageLoan::~StageLoan() {
+    {
+        std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        ctx->stage_free.push_back(stage);
+    }
+    ctx->q_cv.notify_all();
+}
 
 // ---- reading one block -------------------------------------------------------
 
@@ -383,10 +409,14 @@ struct Worker {
         ctx->q_cv.notify_all();
     }
 
-    // One O_DIRECT pread covers a run of consecutive blocks of one request (large
-    // requests amortise the per-request latency of the storage); the blocks then
-    // go through the ring one by one.  Returns false when the file turned out
-    // not to support O_DIRECT and the run has to be read buffered.
+    // One O_DIRECT pread covers a run of consecutive blocks of one request: the storage
+    // serves one very large sequential request faster than the same bytes in pieces
+    // (measured on a virtio disk: 5.2 GB/s with 64 MiB requests, 7.0 GB/s with 1 GiB).
+    // The bytes land in a staging buffer; the blocks are then put on the `staged` queue,
+    // where every idle worker helps to move them through the ring, so the copy of a
+    // large run is spread over all threads and the next read starts at once.  Returns
+    // false when the file turned out not to support O_DIRECT and the run has to be read
+    // buffered.  Blocks that failed are reported in `status`; staged ones are marked 1.
     bool do_direct(std::vector<Block> &run, std::vector<int64_t> &status) {
         FileEntry &f = *run.front().req->file;
         const uint64_t window = align_down(run.front().file_off, kPage);
@@ -414,20 +444,41 @@ struct Worker {
             return false;
         }
         ctx->ctr.read_ns.fetch_add(t1 - t0, std::memory_order_relaxed);
+        std::shared_ptr<StageLoan> loan = std::make_shared<StageLoan>(ctx, stage);
+        stage = nullptr; // the loan returns it
+        std::vector<Staged> ready;
+        ready.reserve(run.size());
         for (size_t i = 0; i < run.size(); ++i) {
             const Block &b = run[i];
             if (got < 0) { status[i] = got; continue; }
             if (window + (uint64_t)got < b.file_off + b.len) { status[i] = -FSTX_E_SHORT_READ; continue; }
-            Slot *slot = nullptr;
-            if ((status[i] = take_slot(&slot)) < 0) continue;
-            uint64_t t2 = now_ns();
-            std::memcpy(slot->host, stage + (b.file_off - window), b.len);
-            ctx->ctr.stage_ns.fetch_add(now_ns() - t2, std::memory_order_relaxed);
-            ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
-            status[i] = ship(b, *slot, 0);
+            status[i] = 1;
+            ready.push_back(Staged{b, loan->stage + (b.file_off - window), loan});
         }
-        return_stage();
-        return true;
+        if (!ready.empty()) {
+            {
+                std::lock_guard<std::mutex> lk(ctx->q_mutex);
+                for (Staged &st : ready) ctx->staged.push_back(std::move(st));
+            }
+            ctx->q_cv.notify_all();
+        }
+        return true; // `loan` drops here; the staged blocks keep the buffer alive
+    }
+
+    // staging buffer -> ring slot -> device, for one block another read left behind
+    void ship_staged(Staged &st) {
+        const Block &b = st.block;
+        int64_t status = b.req->error.load(std::memory_order_relaxed);
+        Slot *slot = nullptr;
+        if (status == 0 && (status = take_slot(&slot)) == 0) {
+            uint64_t t0 = now_ns();
+            std::memcpy(slot->host, st.bytes, b.len);
+            ctx->ctr.stage_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
+            ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
+            status = ship(b, *slot, 0);
+        }
+        st.loan.reset(); // outside q_mutex: the last one hands the buffer back
+        finish(b, status < 0 ? status : 0);
     }
 
     // called with q_mutex held: borrow a staging block, making one if the pool may still grow
@@ -438,8 +489,14 @@ struct Worker {
             return true;
         }
         if (ctx->stage_made >= ctx->stage_max) return false;
+        // address space only: pages become resident as reads touch them, in huge pages where
+        // the system allows (a read into fresh 4 KiB pages spends most of its time faulting)
         void *p = nullptr;
-        if (posix_memalign(&p, kPage, ctx->direct_bytes + 2 * kPage) != 0) p = nullptr;
+        const uint64_t bytes = ctx->direct_bytes + 2 * kPage;
+        if (posix_memalign(&p, bytes >= (4u << 20) ? (2u << 20) : kPage, bytes) != 0) p = nullptr;
+#ifdef MADV_HUGEPAGE
+        if (p && bytes >= (4u << 20)) (void)madvise(p, bytes, MADV_HUGEPAGE);
+#endif
         stage = static_cast<char *>(p); // nullptr: the read reports ENOMEM
         if (p) ++ctx->stage_made;
         return true;
@@ -466,14 +523,23 @@ struct Worker {
         for (;;) {
             run.clear();
             bool direct = false;
+            Staged todo;
+            bool have_staged = false;
             {
                 // Blocks leave the queue in file order.  A block that needs O_DIRECT is
                 // taken together with its token, under this lock, so that the reads reach
                 // the storage in ascending order too (storage that detects sequential
                 // streams serves them about twice as fast as the same requests shuffled).
+                // Blocks that a read has already staged come first: they hold a staging buffer.
                 std::unique_lock<std::mutex> lk(ctx->q_mutex);
                 for (;;) {
-                    ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty(); });
+                    ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty() || !ctx->staged.empty(); });
+                    if (!ctx->staged.empty()) {
+                        todo = std::move(ctx->staged.front());
+                        ctx->staged.pop_front();
+                        have_staged = true;
+                        break;
+                    }
                     if (ctx->queue.empty()) break; // closing and drained
                     const Block &head = ctx->queue.front();
                     direct = dev_rc == 0 && head.req->error.load(std::memory_order_relaxed) == 0 &&
@@ -484,25 +550,32 @@ struct Worker {
                         borrow_stage();
                         break;
                     }
-                    ctx->q_cv.wait(lk); // tokens or staging blocks are all out: wait for one to come back
+                    // tokens or staging buffers are all out: wait for one to come back, or for staged blocks
+                    ctx->q_cv.wait(lk);
                 }
-                if (ctx->queue.empty()) break;
-                run.push_back(std::move(ctx->queue.front()));
-                ctx->queue.pop_front();
-                if (direct) {
-                    // extend the run with the blocks that follow it in the file
-                    uint64_t bytes = run[0].len + run[0].file_off % kPage;
-                    while (!ctx->queue.empty()) {
-                        const Block &nx = ctx->queue.front();
-                        const Block &last = run.back();
-                        if (nx.req != last.req || nx.file_off != last.file_off + last.len ||
-                            bytes + nx.len > ctx->direct_bytes)
-                            break;
-                        bytes += nx.len;
-                        run.push_back(std::move(ctx->queue.front()));
-                        ctx->queue.pop_front();
+                if (!have_staged) {
+                    if (ctx->queue.empty()) break;
+                    run.push_back(std::move(ctx->queue.front()));
+                    ctx->queue.pop_front();
+                    if (direct) {
+                        // extend the run with the blocks that follow it in the file
+                        uint64_t bytes = run[0].len + run[0].file_off % kPage;
+                        while (!ctx->queue.empty()) {
+                            const Block &nx = ctx->queue.front();
+                            const Block &last = run.back();
+                            if (nx.req != last.req || nx.file_off != last.file_off + last.len ||
+                                bytes + nx.len > ctx->direct_bytes)
+                                break;
+                            bytes += nx.len;
+                            run.push_back(std::move(ctx->queue.front()));
+                            ctx->queue.pop_front();
+                        }
                     }
                 }
+            }
+            if (have_staged) {
+                ship_staged(todo);
+                continue;
             }
             // once a request has failed, its remaining blocks are only counted off
             if (dev_rc < 0 || run[0].req->error.load(std::memory_order_relaxed) != 0) {
@@ -516,7 +589,8 @@ struct Worker {
             if (direct) {
                 status.assign(run.size(), 0);
                 if (do_direct(run, status)) {
-                    for (size_t i = 0; i < run.size(); ++i) finish(run[i], status[i]);
+                    for (size_t i = 0; i < run.size(); ++i)
+                        if (status[i] <= 0) finish(run[i], status[i]); // 1: staged, finished by whoever ships it
                     continue;
                 }
             }
@@ -613,7 +687,7 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (cfg.slots_per_thread == 0) cfg.slots_per_thread = 2;
     const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
     if (cfg.max_direct_reads == 0) cfg.max_direct_reads = adaptive_depth ? g_depth_hint.load() : 1;
-    if (cfg.direct_read_bytes == 0) cfg.direct_read_bytes = 64ull << 20;
+    if (cfg.direct_read_bytes == 0) cfg.direct_read_bytes = 1ull << 30;
     cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
     if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 ||
         cfg.slots_per_thread > 64)
@@ -630,7 +704,8 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     ctx->cfg = cfg;
     ctx->adaptive_depth = adaptive_depth;
     ctx->direct_bytes = cfg.direct_read_bytes;
-    ctx->stage_max = (adaptive_depth ? std::min(cfg.n_threads, 8u) : std::min(cfg.max_direct_reads, cfg.n_threads)) + 2;
+    // one staging buffer per read in flight plus one that is being emptied into the ring meanwhile
+    ctx->stage_max = (adaptive_depth ? std::min(cfg.n_threads, 8u) : std::min(cfg.max_direct_reads, cfg.n_threads)) + 1;
     ctx->direct_gate.reset(new Gate(cfg.max_direct_reads, std::min(cfg.n_threads, 32u), adaptive_depth));
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
 

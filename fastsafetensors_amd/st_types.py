@@ -10,7 +10,6 @@ because the header validator needs them without importing torch.
 
 from dataclasses import dataclass
 from enum import Enum
-from fractions import Fraction
 from typing import Optional
 
 
@@ -103,7 +102,7 @@ def dtype_bits(dtype: DType) -> int:
 
 def dtype_size(dtype: DType) -> float:
     """Bytes per logical element, fractional for sub-byte dtypes (0.5 for F4)."""
-    return float(Fraction(_DTYPE_BITS[dtype], 8))
+    return _DTYPE_BITS[dtype] / 8
 
 
 def dtype_storage_align(dtype: DType) -> int:

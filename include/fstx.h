@@ -66,7 +66,7 @@ typedef struct fstx_config {
     uint32_t slots_per_thread; /* ring slots each worker cycles through (0 = default 2)          */
     uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 1)      */
     uint64_t direct_read_bytes; /* bytes one O_DIRECT pread covers: a run of consecutive blocks,
-                                   multiple of block_bytes (0 = 64 MiB)                          */
+                                   multiple of block_bytes (0 = 1 GiB)                           */
     uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH                                              */
     uint32_t reserved;
 } fstx_config;
