@@ -252,6 +252,9 @@ struct fstx_ctx {
     std::condition_variable q_cv;
     std::deque<Block> queue;
     std::deque<Staged> staged; // read by O_DIRECT, waiting for a worker to ship them (q_mutex)
+    uint64_t queue_pops = 0;               // blocks taken off `queue` so far (q_mutex)
+    uint64_t head_verdict_for = ~0ull;     // value of queue_pops the cached verdict belongs to
+    bool head_wants_direct = false;        // whether the block at the head of `queue` is to be read with O_DIRECT
     bool closing = false;
 
     std::mutex done_mutex;
@@ -532,31 +535,47 @@ struct Worker {
                 // streams serves them about twice as fast as the same requests shuffled).
                 // Blocks that a read has already staged come first: they hold a staging buffer.
                 std::unique_lock<std::mutex> lk(ctx->q_mutex);
+                auto take_staged = [&] {
+                    todo = std::move(ctx->staged.front());
+                    ctx->staged.pop_front();
+                    have_staged = true;
+                };
                 for (;;) {
                     ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty() || !ctx->staged.empty(); });
-                    if (!ctx->staged.empty()) {
-                        todo = std::move(ctx->staged.front());
-                        ctx->staged.pop_front();
-                        have_staged = true;
-                        break;
+                    if (ctx->queue.empty()) {
+                        if (!ctx->staged.empty()) take_staged();
+                        break; // with nothing taken: closing and drained
                     }
-                    if (ctx->queue.empty()) break; // closing and drained
-                    const Block &head = ctx->queue.front();
-                    direct = dev_rc == 0 && head.req->error.load(std::memory_order_relaxed) == 0 &&
-                             wants_direct(head);
-                    if (!direct) break;
+                    // The storage comes first: whenever a token and a staging buffer are free the
+                    // next read starts, even while staged blocks wait -- they are what the other
+                    // workers do meanwhile.  The verdict on the head block (one mincore call) is
+                    // kept until that block leaves the queue.
+                    if (ctx->head_verdict_for != ctx->queue_pops) {
+                        const Block &head = ctx->queue.front();
+                        ctx->head_wants_direct = dev_rc == 0 && head.req->error.load(std::memory_order_relaxed) == 0 &&
+                                                 wants_direct(head);
+                        ctx->head_verdict_for = ctx->queue_pops;
+                    }
+                    direct = ctx->head_wants_direct;
+                    if (!direct) break; // a page-cache block: read it now
                     if ((!ctx->stage_free.empty() || ctx->stage_made < ctx->stage_max) &&
                         ctx->direct_gate->try_enter()) {
                         borrow_stage();
                         break;
                     }
-                    // tokens or staging buffers are all out: wait for one to come back, or for staged blocks
+                    direct = false;
+                    if (!ctx->staged.empty()) {
+                        take_staged();
+                        break;
+                    }
+                    // tokens or staging buffers are all out and nothing is staged: wait for either
                     ctx->q_cv.wait(lk);
                 }
                 if (!have_staged) {
                     if (ctx->queue.empty()) break;
                     run.push_back(std::move(ctx->queue.front()));
                     ctx->queue.pop_front();
+                    ++ctx->queue_pops;
                     if (direct) {
                         // extend the run with the blocks that follow it in the file
                         uint64_t bytes = run[0].len + run[0].file_off % kPage;
@@ -569,6 +588,7 @@ struct Worker {
                             bytes += nx.len;
                             run.push_back(std::move(ctx->queue.front()));
                             ctx->queue.pop_front();
+                            ++ctx->queue_pops;
                         }
                     }
                 }
