@@ -59,8 +59,13 @@ def inputs_for(src: str) -> torch.Tensor:
 
 @pytest.mark.parametrize("src,dst", PAIRS)
 def test_convert_matches_torch(src, dst):
-    x = inputs_for(src).to(DEV)
+    x_host = inputs_for(src)
+    x = x_host.to(DEV)
     want = x.to(T[dst])
+    # torch's CPU conversion is a second, independent implementation of the same contract
+    nan = torch.isnan(x_host)
+    isz_ = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[T[dst].itemsize]
+    assert torch.equal(want.cpu().view(isz_)[~nan], x_host.to(T[dst]).view(isz_)[~nan]), "torch CPU and GPU conversions disagree"
     isz = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[T[dst].itemsize]
     n = x.numel()
     # aligned; element-misaligned source (still 16-byte loads); element-misaligned destination
