@@ -430,6 +430,28 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     out["row_block_copy"] = measure(
         launches[0], f"C4 Llama-2-13B bf16 TP=4, row cuts of file 1 of 3: {len(specs) - n1} tensors per rank in "
                      f"{len(launches[0]) // world} launches (contiguous spans, realign_kernel without shift)")
+    # column cuts written straight into a joined tensor (strided destination): the down_proj
+    # column blocks of every layer of the file side by side, per rank
+    downs = [s for s in specs if s.name.endswith("down_proj.weight")]
+    rows, cols = downs[0].shape
+    blk = -(-cols // world)
+    joined = [torch.empty((rows, blk * len(downs)), dtype=torch.int16, device=dev) for _ in range(world)]
+    jjobs = [[(joined[r].data_ptr() + 2 * blk * i, srcs[s.name].data_ptr() + 2 * r * blk, rows, 2 * blk, 2 * cols,
+               2 * blk * len(downs)) for i, s in enumerate(downs)] for r in range(world)]
+    for r in range(world):
+        _native.slice_copy2d_batch(jjobs[r], stream)
+    jt = timed([lambda r=r: _native.slice_copy2d_batch(jjobs[r], stream) for r in range(world)] * max(1, steps))
+    jb = 2 * joined[0].numel() * 2
+    for r in range(world):
+        if not torch.equal(joined[r], torch.cat([srcs[s.name][:, r * blk : (r + 1) * blk] for s in downs], dim=1)):
+            raise SystemExit("bench: joined column blocks differ from slicing + cat")
+    out["slice_join_columns"] = {
+        "workload": f"C4 down_proj [{rows}, {cols}] column blocks of {len(downs)} layers cut into one joined [{rows}, {blk * len(downs)}] "
+                    f"tensor per rank ({-(-len(downs) // 24)} launches of slice2d_kernel per rank)",
+        "launches_timed": len(jt), "avg_launch_ms": sum(jt) / len(jt), "bytes_per_launch": jb,
+        "achieved_GBps": jb / 1e6 / (sum(jt) / len(jt)),
+    }
+    del joined
     # parity at full size: the four ranks' blocks put side by side give the tensor back
     for s in specs:
         dim = ck.llama_shard_dim(s.name)

@@ -80,6 +80,17 @@ class FstxSliceDesc(ctypes.Structure):
     ]
 
 
+class FstxSlice2dDesc(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("src", ctypes.c_void_p),
+        ("outer", ctypes.c_uint64),
+        ("seg_bytes", ctypes.c_uint64),
+        ("src_pitch", ctypes.c_uint64),
+        ("dst_pitch", ctypes.c_uint64),
+    ]
+
+
 class FstxConvertDesc(ctypes.Structure):
     _fields_ = [
         ("dst", ctypes.c_void_p),
@@ -126,6 +137,8 @@ _SIGNATURES = {
     ),
     "fstx_slice_copy_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxSliceDesc), ctypes.c_uint32, ctypes.c_void_p]),
+    "fstx_slice_copy2d_batch": (
+        ctypes.c_int, [ctypes.POINTER(FstxSlice2dDesc), ctypes.c_uint32, ctypes.c_void_p]),
     "fstx_convert_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxConvertDesc), ctypes.c_uint32, ctypes.c_void_p]),
 }
@@ -297,6 +310,14 @@ def slice_copy_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int
         part = jobs[i : i + FSTX_BATCH_MAX]
         arr = (FstxSliceDesc * len(part))(*[FstxSliceDesc(*j) for j in part])
         _check("fstx_slice_copy_batch", lib().fstx_slice_copy_batch(arr, len(part), stream))
+
+
+def slice_copy2d_batch(jobs: Sequence[Tuple[int, int, int, int, int, int]], stream: int = 0) -> None:
+    """``jobs`` = (dst, src, outer, seg_bytes, src_pitch, dst_pitch) tuples; any count."""
+    for i in range(0, len(jobs), FSTX_BATCH_MAX):
+        part = jobs[i : i + FSTX_BATCH_MAX]
+        arr = (FstxSlice2dDesc * len(part))(*[FstxSlice2dDesc(*j) for j in part])
+        _check("fstx_slice_copy2d_batch", lib().fstx_slice_copy2d_batch(arr, len(part), stream))
 
 
 def convert_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:

@@ -76,19 +76,28 @@ struct alignas(32) SliceJob {
 constexpr uint32_t kOwnerSlots = 2048;
 
 typedef uint32_t v8u __attribute__((ext_vector_type(8)));
+typedef uint32_t v16u __attribute__((ext_vector_type(16)));
 
+// Kernel arguments are limited to 4 KiB: 48 jobs of 32 bytes or 24 jobs of 64 bytes fit
+// next to the two lookup tables.
 template <typename Job>
 struct JobTable {
-    Job job[FSTX_BATCH_MAX];
-    uint32_t first_block[FSTX_BATCH_MAX]; // first workgroup of each job (granule aligned)
-    uint32_t owner[kOwnerSlots / 4];      // one byte per granule: index into job[]
+    static_assert(sizeof(Job) == 32 || sizeof(Job) == 64, "jobs are fetched as eight or sixteen dwords");
+    static constexpr uint32_t kJobs = sizeof(Job) == 32 ? FSTX_BATCH_MAX : FSTX_BATCH_MAX / 2;
+    Job job[kJobs];
+    uint32_t first_block[kJobs];     // first workgroup of each job (granule aligned)
+    uint32_t owner[kOwnerSlots / 4]; // one byte per granule: index into job[]
 
-    // the whole 32-byte job in one scalar load
+    // the whole job in one scalar load
     __device__ __forceinline__ Job fetch(uint32_t ji) const {
-        static_assert(sizeof(Job) == 32, "jobs are fetched as eight dwords");
-        const v8u raw = *reinterpret_cast<const v8u *>(&job[ji]);
         Job out;
-        __builtin_memcpy(&out, &raw, sizeof out);
+        if constexpr (sizeof(Job) == 32) {
+            const v8u raw = *reinterpret_cast<const v8u *>(&job[ji]);
+            __builtin_memcpy(&out, &raw, sizeof out);
+        } else {
+            const v16u raw = *reinterpret_cast<const v16u *>(&job[ji]);
+            __builtin_memcpy(&out, &raw, sizeof out);
+        }
         return out;
     }
 };
@@ -237,6 +246,44 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     case 2: slice_units<uint32_t>(job, u); break;
     case 1: slice_units<uint16_t>(job, u); break;
     default: slice_units<uint8_t>(job, u); break;
+    }
+}
+
+// The same gather with a strided destination: segment `row` is written to
+// dst + row * dst_pitch.  Used to cut the blocks of several tensors straight into one
+// joined tensor along an inner dimension.
+struct alignas(64) Slice2dJob {
+    char *dst;
+    const char *src;
+    uint64_t src_pitch, dst_pitch;
+    uint32_t seg_units, total_units, unit_log2, pad0;
+    uint64_t pad1, pad2;
+};
+
+template <typename Unit>
+__device__ __forceinline__ void slice2d_units(const Slice2dJob &job, uint32_t u) {
+    const uint32_t row = u / job.seg_units;
+    const uint32_t col = u - row * job.seg_units;
+    const Unit *src = reinterpret_cast<const Unit *>(job.src + (uint64_t)row * job.src_pitch) + col;
+    Unit *dst = reinterpret_cast<Unit *>(job.dst + (uint64_t)row * job.dst_pitch) + col;
+    st_stream(ld_stream(src), dst);
+}
+
+__global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t granule_log2,
+                                                          const JobTable<Slice2dJob> t) {
+    const uint32_t b = blockIdx.x;
+    const uint32_t ji = find_job(t, granule_log2, b);
+    const Slice2dJob job = t.fetch(ji);
+    const uint32_t lb = b - t.first_block[ji];
+    const uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
+    if (u64 >= job.total_units) return;
+    const uint32_t u = (uint32_t)u64;
+    switch (job.unit_log2) { // uniform across the workgroup
+    case 4: slice2d_units<v4u>(job, u); break;
+    case 3: slice2d_units<uint64_t>(job, u); break;
+    case 2: slice2d_units<uint32_t>(job, u); break;
+    case 1: slice2d_units<uint16_t>(job, u); break;
+    default: slice2d_units<uint8_t>(job, u); break;
     }
 }
 
@@ -713,6 +760,62 @@ extern "C" int fstx_slice_copy(void *dst, const void *src, uint64_t outer, uint6
                                uint64_t src_pitch, void *stream) {
     fstx_slice_desc d{dst, src, outer, seg_bytes, src_pitch};
     return fstx_slice_copy_batch(&d, 1, stream);
+}
+
+extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t n, void *stream) {
+    if (n == 0) return 0;
+    if (!descs) return -FSTX_E_INVAL;
+    if (n > FSTX_BATCH_MAX) return -FSTX_E_TOO_MANY;
+    JobTable<Slice2dJob> t;
+    constexpr uint32_t kJobs = JobTable<Slice2dJob>::kJobs;
+    uint64_t blocks_of[kJobs];
+    uint64_t blocks = 0;
+    uint32_t k = 0;
+    auto flush = [&]() -> int {
+        if (k == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
+        hipLaunchKernelGGL(slice2d_kernel, dim3((uint32_t)grid), dim3(kBlock), 0,
+                           static_cast<hipStream_t>(stream), gl, t);
+        k = 0;
+        blocks = 0;
+        return fstx_internal::check_launch("slice2d_kernel");
+    };
+    fstx_slice_desc dense[FSTX_BATCH_MAX];
+    uint32_t n_dense = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const fstx_slice2d_desc &d = descs[i];
+        if (d.outer == 0 || d.seg_bytes == 0) continue;
+        if (!d.dst || !d.src) return -FSTX_E_INVAL;
+        if (d.outer > 1 && (d.src_pitch < d.seg_bytes || d.dst_pitch < d.seg_bytes)) return -FSTX_E_INVAL;
+        if (d.outer == 1 || d.dst_pitch == d.seg_bytes) {
+            // a dense destination: the plain slice extract (and its LDS and span forms) serves it
+            dense[n_dense++] = fstx_slice_desc{d.dst, d.src, d.outer, d.seg_bytes, d.src_pitch};
+            continue;
+        }
+        const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
+                                             d.src_pitch | d.dst_pitch | 16u);
+        const uint64_t seg_units = d.seg_bytes >> ul;
+        uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
+        if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 4 Gi units or more
+        for (uint64_t row = 0; row < d.outer; row += rows_per_job) {
+            const uint64_t rows = d.outer - row < rows_per_job ? d.outer - row : rows_per_job;
+            const uint64_t units = rows * seg_units;
+            if (k == kJobs || blocks + blocks_for(units) > kMaxBlocksPerLaunch) {
+                int rc = flush();
+                if (rc < 0) return rc;
+            }
+            t.job[k] = Slice2dJob{static_cast<char *>(d.dst) + row * d.dst_pitch,
+                                  static_cast<const char *>(d.src) + row * d.src_pitch,
+                                  d.src_pitch, d.dst_pitch, (uint32_t)seg_units, (uint32_t)units, ul, 0, 0, 0};
+            blocks_of[k] = blocks_for(units);
+            blocks += blocks_of[k];
+            ++k;
+        }
+    }
+    int rc = flush();
+    if (rc < 0) return rc;
+    return n_dense ? fstx_slice_copy_batch(dense, n_dense, stream) : 0;
 }
 
 extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {

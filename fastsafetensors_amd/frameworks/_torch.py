@@ -358,19 +358,20 @@ class TorchOp(FrameworkOpBase):
         if not items or not all(src.real_tensor.is_cuda for src, _ in items):
             return None
         geoms = [self.shard_geometry(frame, dim, rank, world) for _, frame in items]
-        if any(g[1] != 1 for g in geoms):  # blocks are not contiguous in the joined tensor
-            return None
         first_src, first_frame = items[0]
         shape = list(geoms[0][0])
         shape[dim] = sum(g[0][dim] for g in geoms)
         out = self.get_empty_tensor(shape, first_frame.dtype, first_src.device)
+        # every block is `outer` segments; in the joined tensor the segments of one row sit
+        # side by side, so a block's segments are one joined row apart
+        joined_row = sum(g[2] for g in geoms)
         jobs, at = [], out.data_ptr()
         for (src, _), (_, outer, seg, pitch, first) in zip(items, geoms):
-            if seg:
-                jobs.append((at, src.data_ptr() + first, 1, seg, pitch))
+            if seg and outer:
+                jobs.append((at, src.data_ptr() + first, outer, seg, pitch, joined_row))
             at += seg
         if jobs:
-            _native.slice_copy_batch(jobs, torch.cuda.current_stream(first_src.real_tensor.device).cuda_stream)
+            _native.slice_copy2d_batch(jobs, torch.cuda.current_stream(first_src.real_tensor.device).cuda_stream)
         return out
 
     # ---- misc ------------------------------------------------------------------

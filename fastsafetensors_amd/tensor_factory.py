@@ -163,9 +163,9 @@ class LazyTensorFactory:
     def shuffle_multi_cols(self, pg: ProcessGroupBase, tensor_names: List[str], dim: int) -> TensorBase:
         """The rank's blocks of several tensors joined along ``dim``
         (``tensor_factory.py:194-259``).  The blocks are cut straight into their places in
-        the joined tensor by one batched launch when they are contiguous there (``dim``
-        is the outermost dimension with more than one entry); otherwise they are cut
-        first and concatenated afterwards."""
+        the joined tensor by one batched launch (a strided destination when ``dim`` is an
+        inner dimension); cutting first and concatenating afterwards remains only for
+        tensors that are not in GPU memory."""
         frames = []
         ref_shape: Optional[List[int]] = None
         for name in tensor_names:

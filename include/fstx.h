@@ -198,6 +198,23 @@ typedef struct fstx_slice_desc {
  * file_buffer.py:238-259). */
 int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, void *stream);
 
+typedef struct fstx_slice2d_desc {
+    void *dst;
+    const void *src;
+    uint64_t outer;
+    uint64_t seg_bytes;
+    uint64_t src_pitch;
+    uint64_t dst_pitch; /* bytes between segment starts in dst, >= seg_bytes */
+} fstx_slice2d_desc;
+
+/* As fstx_slice_copy_batch, but the o-th segment is written to dst + o*dst_pitch: the
+ * rank's blocks of several tensors land side by side along an inner dimension of one
+ * joined tensor (dst_pitch = the joined row, dst = the joined tensor + the bytes of the
+ * blocks before this one).  Replaces the per-tensor t[slices].contiguous() followed by
+ * torch.cat of LazyTensorFactory.shuffle_multi_cols (tensor_factory.py:194-259) when the
+ * join runs along a dimension that is not the outermost.  n <= FSTX_BATCH_MAX. */
+int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t n, void *stream);
+
 /* element types of fstx_convert_batch */
 enum fstx_elem_type {
     FSTX_F64 = 0,

@@ -249,6 +249,42 @@ def test_slice_lds_random_geometry_in_one_batch(dev):
             assert (dst[outer * seg :] == 201).all(), "wrote past the end"
 
 
+def test_slice2d_strided_destination(dev):
+    """Blocks of several tensors cut straight into one joined tensor along an inner
+    dimension: random geometry (every unit size from 1 to 16 bytes), against torch.cat
+    of torch's own slices; bytes between the blocks' columns stay untouched."""
+    rng = np.random.default_rng(5)
+    for trial in range(12):
+        item = int(rng.choice([1, 2, 4]))
+        dtype = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[item]
+        rows = int(rng.integers(1, 300))
+        n_src = int(rng.integers(1, 30))  # more than 24 jobs: two launches
+        world = int(rng.integers(1, 5))
+        rank = int(rng.integers(0, world))
+        srcs = [torch.randint(0, 120, (rows, int(rng.integers(1, 200)) * int(rng.choice([1, 1, 4, 8]))), dtype=dtype, device=dev)
+                for _ in range(n_src)]
+        parts = []
+        for t in srcs:
+            block = -(-t.shape[1] // world)
+            parts.append(t[:, rank * block : (rank + 1) * block])
+        want = torch.cat(parts, dim=1)
+        out = torch.full((rows, want.shape[1] + 3), 77, dtype=dtype, device=dev)  # 3 guard columns per row
+        jobs, at = [], out.data_ptr()
+        for t, p in zip(srcs, parts):
+            block = -(-t.shape[1] // world)
+            jobs.append((at, t.data_ptr() + min(rank * block, t.shape[1]) * item, rows, p.shape[1] * item,
+                         t.shape[1] * item, out.shape[1] * item))
+            at += p.shape[1] * item
+        _native.slice_copy2d_batch(jobs, stream())
+        assert torch.equal(out[:, : want.shape[1]], want), trial
+        assert (out[:, want.shape[1] :] == 77).all(), "wrote outside the blocks"
+    # argument checks
+    a = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    lib = _native.lib()
+    bad = (_native.FstxSlice2dDesc * 1)(_native.FstxSlice2dDesc(a.data_ptr(), a.data_ptr() + 2048, 4, 64, 128, 32))
+    assert lib.fstx_slice_copy2d_batch(bad, 1, None) == -10001  # dst_pitch < seg_bytes
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do

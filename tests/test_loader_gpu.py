@@ -204,7 +204,7 @@ def test_as_dict_multi_cols_push_and_auto_free(small_configs):
     block = -(-refs[qkv[0]].shape[0] // world)
     want = torch.cat([refs[k][rank * block : (rank + 1) * block] for k in qkv], dim=0)
     assert torch.equal(joined.cpu().view(torch.int16), want.view(torch.int16))
-    # a join along dim 1 (column blocks side by side) takes the cut-then-concatenate route
+    # a join along dim 1 (column blocks side by side): one launch with a strided destination
     o2 = [f"model.layers.{i}.self_attn.o_proj.weight" for i in (0, 1)]
     joined = bufs.get_multi_cols(o2, dim=1).get_raw()
     block = -(-refs[o2[0]].shape[1] // world)
