@@ -18,7 +18,10 @@ Next to it, on the same line:
 ``roofline``      the slice-extract kernel on HBM-resident Llama-2-13B-shaped
                   tensors (config C4, TP=4, all four ranks in turn), timed with
                   events on the stream the launches go to; ``kernels`` carries the
-                  realign kernel on config C2's data section as well.
+                  other kernels as well (realign on config C2's data section, row
+                  cuts, joined column cuts, odd shapes through LDS, fp32 -> bf16).
+``tp_extract``, ``multi_cols``, ``iterate_weights``, ``downcast_on_load``
+                  the callers around the path, timed through the Python API.
 ``pipeline``      measured ceilings of this box -- O_DIRECT read rate of the same
                   files, pinned host-to-device copy rate, page-cache read rate --
                   and the cold / warm load as fractions of min(read, H2D).
@@ -357,7 +360,7 @@ def bench_iterate_weights(files: List[str], threads: int, verify) -> dict:
 
 
 def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
-    """Event-timed launches of the two kernels on HBM-resident data, through the C ABI."""
+    """Event-timed launches of the kernels on HBM-resident data, through the C ABI."""
     import torch
 
     from fastsafetensors_amd import _native

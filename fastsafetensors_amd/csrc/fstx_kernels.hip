@@ -1,21 +1,26 @@
 // SPDX-License-Identifier: Apache-2.0
 //
-// HBM data-movement kernels of the load path, written for gfx950 (CDNA4):
-// 64-wide wavefronts, 16-byte global loads/stores per lane, no MFMA (there is
-// no arithmetic here; the bound is HBM bandwidth).
+// HBM kernels of the load path, written for gfx950 (CDNA4): 64-wide wavefronts,
+// 16-byte global loads/stores per lane, no MFMA (data movement and element-wise
+// rounding only; the bound is HBM bandwidth).
 //
-//   realign copy  : dst[0:n) = src[0:n) for any byte alignment of src and dst.
-//                   Stands in for gds_device_buffer::memmove of the reference
-//                   (cpp/ext.cpp:606-645: two cudaMemcpy through a temporary).
-//   slice extract : dense copy of `outer` segments read at a fixed pitch.
-//                   Stands in for t[slices].contiguous() per rank in
-//                   LazyTensorFactory.shuffle (tensor_factory.py:168-175).
+//   realign copy   : dst[0:n) = src[0:n) for any byte alignment of src and dst.
+//                    Stands in for gds_device_buffer::memmove of the reference
+//                    (cpp/ext.cpp:606-645: two cudaMemcpy through a temporary).
+//   slice extract  : dense copy of `outer` segments read at a fixed pitch.
+//                    Stands in for t[slices].contiguous() per rank in
+//                    LazyTensorFactory.shuffle (tensor_factory.py:168-175).
+//                    Three forms: direct, strided destination (joins), and
+//                    staged through LDS for shapes that are not 16-byte multiples.
+//   down-cast      : element type conversion towards a narrower type with torch's
+//                    rounding (SafeTensorsMetadata.get_tensors with a dtype,
+//                    common.py:355-375).
 //
-// Both kernels take a table of up to FSTX_BATCH_MAX jobs as a by-value kernel
-// argument, so that the many small tensors of a checkpoint file cost one
+// Every kernel takes a table of jobs as a by-value kernel argument (up to
+// FSTX_BATCH_MAX), so that the many small tensors of a checkpoint file cost one
 // launch.  A workgroup is one wavefront and owns 64 consecutive 16-byte vectors
-// of one job's destination; consecutive lanes touch consecutive vectors, so each
-// wavefront reads and writes contiguous 1 KiB spans.
+// of one job's destination (a 2 KiB tile in the LDS form); consecutive lanes touch
+// consecutive vectors, so each wavefront reads and writes contiguous spans.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>

@@ -4,8 +4,8 @@
  *
  * One shared library (libfstx.so, HIP, gfx950) holds
  *   - the file -> pinned ring -> HBM copy pipeline, and
- *   - the two data-movement kernels that post-process tensors in HBM
- *     (realign copy, slice extract).
+ *   - the kernels that post-process tensors in HBM (realign copy, slice
+ *     extract in its dense, strided-destination and LDS-staged forms, down-cast).
  * Every entry point takes plain pointers and sizes; there are no C++ or torch
  * types in the signatures, so the library binds from ctypes, cgo, JNI or any
  * other FFI.  Each declaration names the interface of the reference
