@@ -439,18 +439,17 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     rows, cols = downs[0].shape
     blk = -(-cols // world)
     joined = [torch.empty((rows, blk * len(downs)), dtype=torch.int16, device=dev) for _ in range(world)]
-    jjobs = [[(joined[r].data_ptr() + 2 * blk * i, srcs[s.name].data_ptr() + 2 * r * blk, rows, 2 * blk, 2 * cols,
-               2 * blk * len(downs)) for i, s in enumerate(downs)] for r in range(world)]
+    jsrcs = [[(srcs[s.name].data_ptr() + 2 * r * blk, 2 * blk, 2 * cols) for s in downs] for r in range(world)]
     for r in range(world):
-        _native.slice_copy2d_batch(jjobs[r], stream)
-    jt = timed([lambda r=r: _native.slice_copy2d_batch(jjobs[r], stream) for r in range(world)] * max(1, steps))
+        _native.join_copy(joined[r].data_ptr(), rows, jsrcs[r], stream)
+    jt = timed([lambda r=r: _native.join_copy(joined[r].data_ptr(), rows, jsrcs[r], stream) for r in range(world)] * max(1, steps))
     jb = 2 * joined[0].numel() * 2
     for r in range(world):
         if not torch.equal(joined[r], torch.cat([srcs[s.name][:, r * blk : (r + 1) * blk] for s in downs], dim=1)):
             raise SystemExit("bench: joined column blocks differ from slicing + cat")
     out["slice_join_columns"] = {
         "workload": f"C4 down_proj [{rows}, {cols}] column blocks of {len(downs)} layers cut into one joined [{rows}, {blk * len(downs)}] "
-                    f"tensor per rank ({-(-len(downs) // 24)} launches of slice2d_kernel per rank)",
+                    f"tensor per rank (one launch of join_kernel per rank)",
         "launches_timed": len(jt), "avg_launch_ms": sum(jt) / len(jt), "bytes_per_launch": jb,
         "achieved_GBps": jb / 1e6 / (sum(jt) / len(jt)),
     }

@@ -91,6 +91,10 @@ class FstxSlice2dDesc(ctypes.Structure):
     ]
 
 
+class FstxJoinSrc(ctypes.Structure):
+    _fields_ = [("src", ctypes.c_void_p), ("seg_bytes", ctypes.c_uint64), ("src_pitch", ctypes.c_uint64)]
+
+
 class FstxConvertDesc(ctypes.Structure):
     _fields_ = [
         ("dst", ctypes.c_void_p),
@@ -139,6 +143,9 @@ _SIGNATURES = {
         ctypes.c_int, [ctypes.POINTER(FstxSliceDesc), ctypes.c_uint32, ctypes.c_void_p]),
     "fstx_slice_copy2d_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxSlice2dDesc), ctypes.c_uint32, ctypes.c_void_p]),
+    "fstx_join_copy": (
+        ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.POINTER(FstxJoinSrc), ctypes.c_uint32,
+                       ctypes.c_void_p]),
     "fstx_convert_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxConvertDesc), ctypes.c_uint32, ctypes.c_void_p]),
 }
@@ -318,6 +325,21 @@ def slice_copy2d_batch(jobs: Sequence[Tuple[int, int, int, int, int, int]], stre
         part = jobs[i : i + FSTX_BATCH_MAX]
         arr = (FstxSlice2dDesc * len(part))(*[FstxSlice2dDesc(*j) for j in part])
         _check("fstx_slice_copy2d_batch", lib().fstx_slice_copy2d_batch(arr, len(part), stream))
+
+
+FSTX_JOIN_MAX = 24
+
+
+def join_copy(dst: int, rows: int, srcs: Sequence[Tuple[int, int, int]], stream: int = 0, dst_pitch: int = 0) -> None:
+    """Row r of ``dst`` = the r-th segments of ``srcs`` = (src, seg_bytes, src_pitch) side by
+    side; rows ``dst_pitch`` bytes apart (0: dense).  Any number of sources."""
+    pitch = dst_pitch or sum(s[1] for s in srcs)
+    at = dst
+    for i in range(0, len(srcs), FSTX_JOIN_MAX):
+        part = srcs[i : i + FSTX_JOIN_MAX]
+        arr = (FstxJoinSrc * len(part))(*[FstxJoinSrc(*s) for s in part])
+        _check("fstx_join_copy", lib().fstx_join_copy(at, pitch, rows, arr, len(part), stream))
+        at += sum(s[1] for s in part)
 
 
 def convert_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:

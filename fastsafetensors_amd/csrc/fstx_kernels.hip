@@ -292,6 +292,58 @@ __global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t granule_
     }
 }
 
+// Fused slice + concatenate along an inner dimension.  The destination is swept in row
+// order: a chunk is `rows_per_chunk` rows of the joined tensor, and within a chunk the
+// sources follow one another, each with whole wavefronts of its own (a wavefront never
+// mixes sources, so everything that selects the source is scalar work).  Writes therefore
+// stay within a few hundred KB of one another instead of striding through the whole
+// destination once per source.
+struct alignas(32) JoinSrc {
+    const char *src;     // the block's first byte in row 0
+    uint64_t src_pitch;
+    uint32_t seg_units;  // units per row
+    uint32_t dst_col;    // byte offset of the block in a joined row
+    uint64_t pad;
+};
+
+struct JoinTable {
+    char *dst;
+    uint64_t dst_pitch;       // bytes of a joined row
+    uint32_t rows, rows_per_chunk, waves_per_chunk, n, unit_log2;
+    uint32_t wave_begin[FSTX_JOIN_MAX]; // first wavefront of each source within a chunk
+    JoinSrc src[FSTX_JOIN_MAX];
+};
+
+template <typename Unit>
+__device__ __forceinline__ void join_units(const JoinTable &t, const JoinSrc &js, uint32_t chunk, uint32_t u) {
+    const uint32_t r = u / js.seg_units;
+    const uint32_t col = u - r * js.seg_units;
+    const uint64_t row = (uint64_t)chunk * t.rows_per_chunk + r;
+    if (r >= t.rows_per_chunk || row >= t.rows) return; // idle lanes at the end of a source's share
+    const Unit *src = reinterpret_cast<const Unit *>(js.src + row * js.src_pitch) + col;
+    Unit *dst = reinterpret_cast<Unit *>(t.dst + row * t.dst_pitch + js.dst_col) + col;
+    st_stream(ld_stream(src), dst);
+}
+
+__global__ __launch_bounds__(kBlock) void join_kernel(const JoinTable t) {
+    const uint32_t b = blockIdx.x;
+    const uint32_t chunk = b / t.waves_per_chunk;
+    const uint32_t w = b - chunk * t.waves_per_chunk;
+    uint32_t k = 0;
+    for (uint32_t j = 1; j < t.n; ++j) k += w >= t.wave_begin[j] ? 1u : 0u; // uniform: scalar compares
+    const v8u raw = *reinterpret_cast<const v8u *>(&t.src[k]);
+    JoinSrc js;
+    __builtin_memcpy(&js, &raw, sizeof js);
+    const uint32_t u = (w - t.wave_begin[k]) * kBlock + threadIdx.x;
+    switch (t.unit_log2) { // uniform across the launch
+    case 4: join_units<v4u>(t, js, chunk, u); break;
+    case 3: join_units<uint64_t>(t, js, chunk, u); break;
+    case 2: join_units<uint32_t>(t, js, chunk, u); break;
+    case 1: join_units<uint16_t>(t, js, chunk, u); break;
+    default: join_units<uint8_t>(t, js, chunk, u); break;
+    }
+}
+
 // ------------------------------------- slice extract, staged through LDS
 //
 // For segments whose length, pitch or source address is not a multiple of 16
@@ -821,6 +873,55 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
     int rc = flush();
     if (rc < 0) return rc;
     return n_dense ? fstx_slice_copy_batch(dense, n_dense, stream) : 0;
+}
+
+extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,
+                              void *stream) {
+    if (n == 0 || rows == 0) return 0;
+    if (!dst || !srcs) return -FSTX_E_INVAL;
+    if (n > FSTX_JOIN_MAX) return -FSTX_E_TOO_MANY;
+    JoinTable t{};
+    t.dst = static_cast<char *>(dst);
+    uint64_t bits = (uint64_t)(uintptr_t)dst | 16u, row_bytes = 0, min_seg = ~0ull;
+    for (uint32_t i = 0; i < n; ++i) {
+        const fstx_join_src &s = srcs[i];
+        if (s.seg_bytes == 0) continue;
+        if (!s.src || (rows > 1 && s.src_pitch < s.seg_bytes) || s.seg_bytes >> 32) return -FSTX_E_INVAL;
+        bits |= (uint64_t)(uintptr_t)s.src | s.seg_bytes | s.src_pitch;
+        row_bytes += s.seg_bytes;
+        if (s.seg_bytes < min_seg) min_seg = s.seg_bytes;
+    }
+    if (row_bytes == 0) return 0;
+    if (dst_pitch == 0) dst_pitch = row_bytes;
+    if (dst_pitch < row_bytes) return -FSTX_E_INVAL;
+    if (row_bytes >> 32 || rows >> 32) return -FSTX_E_RANGE;
+    const uint32_t ul = common_unit_log2(bits | dst_pitch);
+    t.dst_pitch = dst_pitch;
+    t.rows = (uint32_t)rows;
+    t.unit_log2 = ul;
+    // rows per chunk: the shortest block still fills sixteen wavefronts, so that the idle
+    // lanes at the end of each source's share of a chunk stay below a few percent
+    uint64_t rpc = (16ull * kBlock + (min_seg >> ul) - 1) / (min_seg >> ul);
+    if (rpc > rows) rpc = rows;
+    t.rows_per_chunk = (uint32_t)rpc;
+    uint64_t waves = 0, col = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const fstx_join_src &s = srcs[i];
+        if (s.seg_bytes == 0) continue;
+        const uint64_t units = rpc * (s.seg_bytes >> ul);
+        if (units > kMaxUnitsPerJob) return -FSTX_E_RANGE;
+        t.wave_begin[t.n] = (uint32_t)waves;
+        t.src[t.n] = JoinSrc{static_cast<const char *>(s.src), s.src_pitch, (uint32_t)(s.seg_bytes >> ul), (uint32_t)col, 0};
+        waves += (units + kBlock - 1) / kBlock;
+        col += s.seg_bytes;
+        ++t.n;
+    }
+    const uint64_t chunks = (rows + rpc - 1) / rpc;
+    if (waves > 0xffffffffull || chunks * waves > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
+    t.waves_per_chunk = (uint32_t)waves;
+    hipLaunchKernelGGL(join_kernel, dim3((uint32_t)(chunks * waves)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), t);
+    return fstx_internal::check_launch("join_kernel");
 }
 
 extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {

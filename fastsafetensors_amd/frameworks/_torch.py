@@ -364,14 +364,22 @@ class TorchOp(FrameworkOpBase):
         out = self.get_empty_tensor(shape, first_frame.dtype, first_src.device)
         # every block is `outer` segments; in the joined tensor the segments of one row sit
         # side by side, so a block's segments are one joined row apart
-        joined_row = sum(g[2] for g in geoms)
-        jobs, at = [], out.data_ptr()
-        for (src, _), (_, outer, seg, pitch, first) in zip(items, geoms):
-            if seg and outer:
-                jobs.append((at, src.data_ptr() + first, outer, seg, pitch, joined_row))
-            at += seg
-        if jobs:
-            _native.slice_copy2d_batch(jobs, torch.cuda.current_stream(first_src.real_tensor.device).cuda_stream)
+        outer = geoms[0][1]
+        stream = torch.cuda.current_stream(first_src.real_tensor.device).cuda_stream
+        if outer == 1:
+            # a join along the outermost dimension: the blocks are contiguous spans of the result
+            jobs, at = [], out.data_ptr()
+            for (src, _), (_, _o, seg, pitch, first) in zip(items, geoms):
+                if seg:
+                    jobs.append((at, src.data_ptr() + first, 1, seg, pitch))
+                at += seg
+            _native.slice_copy_batch(jobs, stream)
+        elif outer and any(g[2] for g in geoms):
+            _native.join_copy(
+                out.data_ptr(), outer,
+                [(src.data_ptr() + first, seg, pitch) for (src, _), (_, _o, seg, pitch, first) in zip(items, geoms)],
+                stream,
+            )
         return out
 
     # ---- misc ------------------------------------------------------------------

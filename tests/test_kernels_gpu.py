@@ -285,6 +285,42 @@ def test_slice2d_strided_destination(dev):
     assert lib.fstx_slice_copy2d_batch(bad, 1, None) == -10001  # dst_pitch < seg_bytes
 
 
+def test_join_copy_matches_cat(dev):
+    """fstx_join_copy: the blocks of up to 60 tensors side by side in one joined tensor,
+    against torch.cat of torch's own slices; every unit size, short and long segments,
+    a padded destination, guard bytes."""
+    rng = np.random.default_rng(9)
+    for trial in range(14):
+        item = int(rng.choice([1, 2, 4]))
+        dtype = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[item]
+        rows = int(rng.integers(1, 400))
+        n_src = int(rng.choice([1, 2, 3, 7, 24, 25, 60]))
+        world = int(rng.integers(1, 5))
+        rank = int(rng.integers(0, world))
+        srcs = [torch.randint(0, 120, (rows, int(rng.integers(1, 300)) * int(rng.choice([1, 1, 4, 8, 64]))), dtype=dtype, device=dev)
+                for _ in range(n_src)]
+        parts = []
+        for t in srcs:
+            block = -(-t.shape[1] // world)
+            parts.append(t[:, min(rank * block, t.shape[1]) : (rank + 1) * block])
+        want = torch.cat(parts, dim=1)
+        pad = int(rng.choice([0, 3, 16]))
+        out = torch.full((rows, want.shape[1] + pad), 77, dtype=dtype, device=dev)
+        jobs = [(t.data_ptr() + (p.storage_offset() - t.storage_offset()) * item, p.shape[1] * item, t.shape[1] * item)
+                for t, p in zip(srcs, parts)]
+        _native.join_copy(out.data_ptr(), rows, jobs, stream(), dst_pitch=out.shape[1] * item)
+        assert torch.equal(out[:, : want.shape[1]], want), trial
+        assert (out[:, want.shape[1] :] == 77).all(), "wrote outside the joined columns"
+    lib = _native.lib()
+    a = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    one = (_native.FstxJoinSrc * 1)(_native.FstxJoinSrc(a.data_ptr() + 2048, 64, 32))
+    assert lib.fstx_join_copy(a.data_ptr(), 0, 4, one, 1, None) == -10001  # pitch shorter than the segment
+    one = (_native.FstxJoinSrc * 1)(_native.FstxJoinSrc(a.data_ptr() + 2048, 64, 64))
+    assert lib.fstx_join_copy(a.data_ptr(), 32, 4, one, 1, None) == -10001  # destination rows would overlap
+    many = (_native.FstxJoinSrc * 25)()
+    assert lib.fstx_join_copy(a.data_ptr(), 0, 4, many, 25, None) == -10008
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do

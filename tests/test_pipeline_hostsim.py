@@ -19,7 +19,7 @@ from fastsafetensors_amd import _native
 HERE = os.path.dirname(os.path.abspath(__file__))
 SIM_DIR = os.path.join(HERE, "hostsim")
 PIPELINE_SYMBOLS = [
-    n for n in _native.EXPORTED_SYMBOLS if not ("realign" in n or "slice" in n or "convert" in n)
+    n for n in _native.EXPORTED_SYMBOLS if not ("realign" in n or "slice" in n or "convert" in n or "join" in n)
 ]
 
 
