@@ -4,10 +4,8 @@ C ABI and the loader, bit for bit against torch's own Tensor.to() on the same de
 (the reference converts with exactly that call, common.py:355-375).  Floating point,
 but the bar is still bit-exact: rounding mode, overflow and NaN handling are part
 of the contract."""
-import itertools
 import os
 
-import numpy as np
 import pytest
 import torch
 from safetensors.torch import load_file
