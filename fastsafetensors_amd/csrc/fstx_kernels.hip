@@ -431,20 +431,42 @@ __device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, 
     uint32_t group_log2 = 6;
     while (group_log2 > 0 && (32u >> (6 - group_log2)) >= vmax) --group_log2;
     const uint32_t group = 1u << group_log2;
-    for (uint32_t ibase = 0; ibase < nrows; ibase += 64u >> group_log2) {
-        const uint32_t i = ibase + (lane >> group_log2);
-        if (i < nrows) {
+    if (group_log2 == 6) {
+        // Long row pieces, one per step: the loads go from global memory straight into LDS
+        // (lane l of an instruction lands at the instruction's LDS base + 16 l), no register
+        // in between, so all loads of the tile are in flight before the first one is waited for.
+        for (uint32_t i = 0; i < nrows; ++i) {
             const uint32_t cb = g.col_begin(i);
             const uint32_t pos_end = (i + 1) * seg < g.end_pos ? (i + 1) * seg : g.end_pos;
             const uintptr_t a0 = (uintptr_t)src_row0 + (uint64_t)i * pitch + cb;
             const uintptr_t a1 = a0 + (pos_end - (i * seg + cb));
             const uintptr_t lo = a0 & ~(uintptr_t)15;
             const uint32_t at = g.slot(i);
-            for (uint32_t v = lane & (group - 1); lo + 16ull * v < a1; v += group)
-                                // a plain load, not a streaming one: the cache lines at the ends of a piece are shared
+            for (uint32_t base = 0; lo + 16ull * base < a1; base += 64) {
+                const uintptr_t mine = lo + 16ull * (base + lane);
+                if (mine < a1)
+                    __builtin_amdgcn_global_load_lds((const FSTX_GLOBAL void *)mine,
+                                                     (__attribute__((address_space(3))) void *)(lds + at + 16 * base),
+                                                     16, 0, 0);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+        for (uint32_t ibase = 0; ibase < nrows; ibase += 64u >> group_log2) {
+            const uint32_t i = ibase + (lane >> group_log2);
+            if (i < nrows) {
+                const uint32_t cb = g.col_begin(i);
+                const uint32_t pos_end = (i + 1) * seg < g.end_pos ? (i + 1) * seg : g.end_pos;
+                const uintptr_t a0 = (uintptr_t)src_row0 + (uint64_t)i * pitch + cb;
+                const uintptr_t a1 = a0 + (pos_end - (i * seg + cb));
+                const uintptr_t lo = a0 & ~(uintptr_t)15;
+                const uint32_t at = g.slot(i);
+                // plain loads, not streaming ones: the cache lines at the ends of a piece are shared
                 // with the neighbouring tile, and streaming lines were fetched from HBM again for it
                 // (fetch traffic 9.6 % over the algorithmic bytes against 3.1 % with plain loads)
-                *reinterpret_cast<v4u *>(lds + at + 16 * v) = ld_global(reinterpret_cast<const v4u *>(lo) + v);
+                for (uint32_t v = lane & (group - 1); lo + 16ull * v < a1; v += group)
+                    *reinterpret_cast<v4u *>(lds + at + 16 * v) = ld_global(reinterpret_cast<const v4u *>(lo) + v);
+            }
         }
     }
     __syncthreads(); // one wavefront: orders its LDS writes before the reads below
