@@ -47,9 +47,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one launch of the roofline workload (slice_kernel, C4 column cuts, 28 tensors) moved
 # according to rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by its reading for an aligned
-# 1 GiB copy (x1.99987 and x0.99966): profiles/fstx_kernels_hbm_traffic_counters.md.  Algorithmic:
+# 1 GiB copy (x1.99987 and x0.99962): profiles/fstx_kernels_hbm_traffic_counters.md.  Algorithmic:
 # 1,357,905,920.
-SLICE_KERNEL_TRAFFIC_BYTES = 1_357_747_979
+SLICE_KERNEL_TRAFFIC_BYTES = 1_357_700_395
 
 
 def log(*a):
