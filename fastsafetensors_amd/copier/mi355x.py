@@ -40,6 +40,7 @@ from .base import CopierInterface
 from .registry import CopierConstructFunc, register_copier_constructor
 
 PTR_ALIGN = 16
+LINE_ALIGN = 128  # tensors placed in side buffers start on cache lines: the copy kernels write whole lines then
 WINDOW_ALIGN = 4096
 LAYOUTS = ("direct", "window")
 
@@ -166,7 +167,7 @@ class MI355XFileCopier(CopierInterface):
             cursor = 0
             for name, frame in need.items():
                 placed[name] = cursor
-                cursor += _align_up(frame.nbytes, PTR_ALIGN)
+                cursor += _align_up(frame.nbytes, LINE_ALIGN)
             side = fw.alloc_side_memory(gbuf, cursor, self.device)
             _native.realign_copy_batch(
                 [
@@ -210,7 +211,7 @@ class MI355XFileCopier(CopierInterface):
             if frame.dtype != dtype or (src_at + frame.data_offsets[0]) % PTR_ALIGN:
                 placed[name] = cursor
                 count = frame.nbytes * 8 // dtype_bits(frame.dtype)
-                cursor += _align_up(count * (want_bits if frame.dtype != dtype else dtype_bits(frame.dtype)) // 8, PTR_ALIGN)
+                cursor += _align_up(count * (want_bits if frame.dtype != dtype else dtype_bits(frame.dtype)) // 8, LINE_ALIGN)
         side = fw.alloc_side_memory(gbuf, cursor, self.device)
         convert, copy = [], []
         for name, at in placed.items():

@@ -179,21 +179,28 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     v4u *dstv = reinterpret_cast<v4u *>(job.dst + head);
     const char *s = job.src + head;
     const uint32_t m = (uint32_t)(uintptr_t)s & (kVecBytes - 1);
-    if (m == 0) {
-        // already aligned: a plain streaming copy, workgroups in dispatch order
-        const uint64_t j = (uint64_t)lb * kBlock + threadIdx.x;
-        const v4u *srcv = reinterpret_cast<const v4u *>(s);
-        if (j < nvec) st_stream(ld_stream(srcv + j), dstv + j);
-        return;
-    }
-    // Workgroups go round-robin over the eight dies, each with its own L2.  Give
-    // each die one contiguous eighth of the job, so that the source vector shared
-    // by two neighbouring wavefronts is fetched from HBM once and found in that
-    // die's L2 the second time (with neighbours on different dies it is fetched twice).
+    // Workgroups go round-robin over the eight dies, each with its own L2.  Whenever the
+    // 1 KiB spans of neighbouring wavefronts share a cache line (source or destination not
+    // on a 128-byte boundary) or a source vector (source shifted), give each die one
+    // contiguous eighth of the job: the shared line is then fetched from HBM once and
+    // found in that die's L2 the second time, and a destination line is completed within
+    // one L2 (with neighbours on different dies it is fetched, or partially written, twice).
     const uint64_t nblocks = (nvec + kBlock - 1) / kBlock;
     const uint64_t per_die = (nblocks + kXcds - 1) / kXcds;
     const uint64_t turn = lb / kXcds;
-    const uint64_t j = ((lb % kXcds) * per_die + turn) * kBlock + threadIdx.x;
+    const uint64_t j_by_die = ((lb % kXcds) * per_die + turn) * kBlock + threadIdx.x;
+    if (m == 0) {
+        // source vectors are aligned: a plain streaming copy; in dispatch order when both
+        // sides sit on cache-line boundaries
+        const bool by_die = ((((uintptr_t)s) | (uintptr_t)dstv) & 127) != 0;
+        const uint64_t j = by_die ? j_by_die : (uint64_t)lb * kBlock + threadIdx.x;
+        const v4u *srcv = reinterpret_cast<const v4u *>(s);
+        if ((!by_die || turn < per_die) && j < nvec) {
+            st_stream(ld_stream(srcv + j), dstv + j);
+        }
+        return;
+    }
+    const uint64_t j = j_by_die;
     const bool live = turn < per_die && j < nvec; // idle workgroups pad a job to whole eighths and granules
     // Source vectors are loaded at their natural 16-byte alignment; output vector j
     // is bytes [m, m+16) of aligned vectors j and j+1.  Every lane loads vector j
@@ -242,7 +249,20 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     const uint32_t ji = find_job(t, granule_log2, b);
     const SliceJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
-    const uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
+    // in dispatch order when every segment starts on a cache-line boundary on both sides,
+    // else one contiguous eighth of the job per die (see realign_kernel)
+    uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
+#ifndef FSTX_SLICE_NO_REMAP
+    const uint32_t ulog = (uint32_t)(job.pitch_unit >> 56);
+    const uint64_t seg_bytes = (uint64_t)job.seg_units << ulog;
+    if ((((uintptr_t)job.dst | (uintptr_t)job.src | job.pitch_unit | seg_bytes) & 127) != 0) {
+        const uint32_t nblocks = (job.total_units + kBlock - 1) / kBlock;
+        const uint32_t per_die = (nblocks + kXcds - 1) / kXcds;
+        const uint32_t turn = lb / kXcds;
+        if (turn >= per_die) return;
+        u64 = ((uint64_t)(lb % kXcds) * per_die + turn) * kBlock + threadIdx.x;
+    }
+#endif
     if (u64 >= job.total_units) return; // also retires the idle workgroups of a job's last granule
     const uint32_t u = (uint32_t)u64;
     switch ((uint32_t)(job.pitch_unit >> 56)) { // uniform across the workgroup
@@ -822,14 +842,14 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         for (uint64_t row = 0; row < outer; row += rows_per_job) {
             uint64_t rows = outer - row < rows_per_job ? outer - row : rows_per_job;
             uint64_t units = rows * seg_units;
-            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) > kMaxBlocksPerLaunch) {
+            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > kMaxBlocksPerLaunch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
             t.job[k] = SliceJob{static_cast<char *>(d.dst) + row * seg,
                                 static_cast<const char *>(d.src) + row * pitch,
                                 pitch | ((uint64_t)ul << 56), (uint32_t)seg_units, (uint32_t)units};
-            blocks_of[k] = blocks_for(units);
+            blocks_of[k] = (blocks_for(units) + kXcds - 1) / kXcds * kXcds; // whole eighths
             blocks += blocks_of[k];
             ++k;
         }
