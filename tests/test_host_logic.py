@@ -208,7 +208,9 @@ def test_pick_lead_prefers_most_bytes():
         return TensorFrame(DType.U8, [n], [start, start + n], [1], [0], False)
 
     assert pick_lead([f(0, 64), f(64, 64)]) == 0
-    assert pick_lead([f(0, 4), f(4, 4), f(8, 1000), f(1008, 16)]) == 8  # the big one starts at 8 -> lead 8
+    assert pick_lead([f(0, 4), f(4, 4), f(8, 1000), f(1008, 16)]) == 120  # the big one starts at 8 -> on a line at 128
+    assert pick_lead([f(0, 4), f(4, 4), f(8, 1000), f(1008, 16)], line=16) == 8
+    assert pick_lead([f(0, 48), f(48, 4096)]) == 80  # 16-byte alignment holds for both at 0, 16, ..; 80 puts the big one on a line
     assert pick_lead([f(0, 10), f(10, 10)]) == 0  # tie -> smallest lead
     assert pick_lead([]) == 0
 
