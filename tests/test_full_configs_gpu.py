@@ -57,7 +57,15 @@ def load_and_check(files, sums, **kw):
     return loader, bufs
 
 
+def need_free(directory: str, nbytes: float) -> None:
+    os.makedirs(directory, exist_ok=True)
+    st = os.statvfs(directory)
+    if st.f_bavail * st.f_frsize < nbytes:
+        pytest.skip(f"{directory} has less than {nbytes / 1e9:.0f} GB free (set FSTX_TEST_DIR)")
+
+
 def test_c3_llama3_8b_full_size(data_dir):
+    need_free(data_dir, 18e9)
     files, sums, nbytes = write_with_checksums("C3", os.path.join(data_dir, "full_C3"))
     assert nbytes == 16_060_522_496 and len(sums) == 291
     try:
@@ -74,6 +82,7 @@ def test_c3_llama3_8b_full_size(data_dir):
 def test_c4_llama2_13b_tp4_full_size(data_dir):
     """All four TP=4 ranks' shards, extracted in turn on one GPU, against torch's own
     slice of the (checksum-verified) whole tensor."""
+    need_free(data_dir, 28e9)
     files, sums, nbytes = write_with_checksums("C4", os.path.join(data_dir, "full_C4"))
     assert nbytes == 26_031_728_640 and len(sums) == 363
     try:
