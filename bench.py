@@ -267,7 +267,7 @@ def bench_tp_extract(files: List[str], world: int, threads: int, block_kb: int) 
     for key, dim in dims.items():
         full = whole.get_tensor(key)
         got = per_rank[0][key] if dim < 0 else torch.cat([per_rank[r][key] for r in range(world)], dim=dim)
-        if got.shape != full.shape or not torch.equal(got.view(torch.uint8), full.view(torch.uint8)):
+        if got.shape != full.shape or not torch.equal(got.reshape(-1).view(torch.uint8), full.reshape(-1).view(torch.uint8)):
             raise SystemExit(f"bench: TP blocks of {key} do not reassemble to the tensor")
         checked += 1
     whole.close()
