@@ -37,6 +37,37 @@ def test_constants_match_the_header():
     assert ctypes.sizeof(_native.FstxCopyDesc) == 24 and ctypes.sizeof(_native.FstxSliceDesc) == 40
 
 
+def test_header_is_plain_c_and_struct_layouts_match_the_binding(tmp_path):
+    """include/fstx.h compiles as C99 on its own, and a C compiler lays the structs out
+    exactly as the ctypes binding does (size and the offset of every field)."""
+    import shutil
+    import subprocess
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    pairs = {"fstx_config": _native.FstxConfig, "fstx_metrics": _native.FstxMetrics, "fstx_copy_desc": _native.FstxCopyDesc,
+             "fstx_slice_desc": _native.FstxSliceDesc, "fstx_slice2d_desc": _native.FstxSlice2dDesc,
+             "fstx_join_src": _native.FstxJoinSrc, "fstx_convert_desc": _native.FstxConvertDesc}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "fstx.h"', "int main(void) {"]
+    for cname, ctype in pairs.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for field, _t in ctype._fields_:
+            lines.append(f'  printf("{cname}.{field} %zu\\n", offsetof({cname}, {field}));')
+    lines += ['  printf("FSTX_JOIN_MAX %d\\n", FSTX_JOIN_MAX);', "  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run([cc, "-std=c99", "-Wall", "-Werror", "-pedantic", f"-I{os.path.join(ROOT, 'include')}", str(src), "-o", str(exe)],
+                   check=True)
+    got = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, ctype in pairs.items():
+        assert int(got[cname]) == ctypes.sizeof(ctype), cname
+        for field, _t in ctype._fields_:
+            assert int(got[f"{cname}.{field}"]) == getattr(ctype, field).offset, (cname, field)
+    assert int(got["FSTX_JOIN_MAX"]) == _native.FSTX_JOIN_MAX
+
+
 def test_host_helpers():
     assert _native.get_alignment_size() == 4096  # reference: tests/smoke_import_cpp.py:34-40
     assert _native.get_cpp_metrics().bounce_buffer_bytes == 0
