@@ -237,9 +237,9 @@ class MI355XFileCopier(CopierInterface):
             if name in placed:
                 if frame.dtype != dtype:
                     count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                    # a frame of its own for the view: the header model keeps describing the file
                     frame = TensorFrame(dtype, frame.shape, [placed[name], placed[name] + count * want_bits // 8],
                                         frame.strides, frame.offsets, frame.sliced)
-                    meta.tensors[name].dtype = dtype  # the header model reports the converted type from now on
                 tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
             else:
                 tensors[name] = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)

@@ -291,12 +291,16 @@ class TorchOp(FrameworkOpBase):
         return tuple(slices[:-1]) + (last,)
 
     # ---- shard extraction ----------------------------------------------------
-    def shard_geometry(self, frame: TensorFrame, dim: int, rank: int, world: int) -> Tuple[List[int], int, int, int, int]:
+    def shard_geometry(
+        self, frame: TensorFrame, dim: int, rank: int, world: int, dtype: Optional[DType] = None
+    ) -> Tuple[List[int], int, int, int, int]:
         """Shape and copy geometry of rank ``rank``'s block of ``frame`` along ``dim``.
 
         Returns ``(shard_shape, outer, seg_bytes, src_pitch, src_byte_offset)`` in
         terms of the tensor's row-major bytes: ``outer`` segments of
         ``seg_bytes``, ``src_pitch`` apart, the first at ``src_byte_offset``.
+        ``dtype`` is the element type the tensor has in memory when that is not the
+        file's any more (a load that converted it).
         """
         shape = frame.shape
         if not 0 <= dim < len(shape):
@@ -305,7 +309,7 @@ class TorchOp(FrameworkOpBase):
         block = -(-extent // world)
         lo = min(rank * block, extent)
         hi = min(lo + block, extent)
-        bits = int(dtype_size(frame.dtype) * 8)
+        bits = int(dtype_size(dtype or frame.dtype) * 8)
         inner_bits = math.prod(shape[dim + 1 :]) * bits
         if (inner_bits * lo) % 8 or (inner_bits * hi) % 8 or (inner_bits * extent) % 8:
             raise ValueError(
@@ -318,8 +322,8 @@ class TorchOp(FrameworkOpBase):
         return out_shape, outer, inner_bits * (hi - lo) // 8, inner_bits * extent // 8, inner_bits * lo // 8
 
     def extract_shard(self, src: TorchTensor, frame: TensorFrame, dim: int, rank: int, world: int) -> TorchTensor:
-        out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world)
-        dst = self.get_empty_tensor(out_shape, frame.dtype, src.device)
+        out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world, src.dtype)
+        dst = self.get_empty_tensor(out_shape, src.dtype, src.device)
         if outer * seg:
             if not src.real_tensor.is_cuda:
                 raise RuntimeError("extract_shard needs a tensor in GPU memory (no CPU path exists)")
@@ -337,10 +341,11 @@ class TorchOp(FrameworkOpBase):
         stream = None
         for src, frame, dim in items:
             if dim == -1:
-                out_shape, outer, seg, pitch, first = list(frame.shape), 1, frame.nbytes, frame.nbytes, 0
+                nbytes = src.real_tensor.numel() * src.real_tensor.element_size()
+                out_shape, outer, seg, pitch, first = list(frame.shape), 1, nbytes, nbytes, 0
             else:
-                out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world)
-            dst = self.get_empty_tensor(out_shape, frame.dtype, src.device)
+                out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world, src.dtype)
+            dst = self.get_empty_tensor(out_shape, src.dtype, src.device)
             outs.append(dst)
             if outer * seg:
                 if not src.real_tensor.is_cuda:
@@ -357,11 +362,11 @@ class TorchOp(FrameworkOpBase):
     ) -> Optional[TorchTensor]:
         if not items or not all(src.real_tensor.is_cuda for src, _ in items):
             return None
-        geoms = [self.shard_geometry(frame, dim, rank, world) for _, frame in items]
+        geoms = [self.shard_geometry(frame, dim, rank, world, src.dtype) for src, frame in items]
         first_src, first_frame = items[0]
         shape = list(geoms[0][0])
         shape[dim] = sum(g[0][dim] for g in geoms)
-        out = self.get_empty_tensor(shape, first_frame.dtype, first_src.device)
+        out = self.get_empty_tensor(shape, first_src.dtype, first_src.device)
         # every block is `outer` segments; in the joined tensor the segments of one row sit
         # side by side, so a block's segments are one joined row apart
         outer = geoms[0][1]

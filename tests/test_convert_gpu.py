@@ -123,10 +123,49 @@ def test_loader_downcast_matches_torch(data_dir, layout):
         if dtype != DType.F32:  # the file now occupies its converted size only
             data = recs[0]["size"] - recs[0]["header_length"]
             assert fw.get_mem_used() < data * tdt.itemsize / 4 + 128 * len(ref) + 64
-            assert loader.frames[next(iter(ref))].dtype == dtype
+            assert loader.frames[next(iter(ref))].dtype == DType.F32  # the header model still describes the file
         bufs.close()
         loader.close()
         assert fw.get_mem_used() == 0
+
+
+def test_shards_and_copies_of_a_downcast_load(data_dir):
+    """After a converting load the tensors in memory are narrower than the file says:
+    rank blocks, whole copies and joins must follow the tensors, not the header."""
+    from collections import OrderedDict
+
+    from fastsafetensors_amd import StubProcessGroup
+
+    recs = ck.write_config(ck.configs(0.06)["C1"], os.path.join(data_dir, "conv_C1"))
+    path = recs[0]["path"]
+    ref = {k: v.to(torch.bfloat16) for k, v in load_file(path, device=DEV).items()}
+    rank, world = 1, 3
+    loader = SafeTensorsFileLoader(StubProcessGroup(rank, world), DEV, max_threads=4)
+    loader.add_filenames({rank: [path]})
+    bufs = loader.copy_files_to_device(dtype=DType.BF16)
+    bufs.auto_mem_delete = False
+    two_d = [k for k, v in ref.items() if v.dim() == 2]
+    same_rows = [k for k in two_d if ref[k].shape[0] == ref[two_d[0]].shape[0]][:3]
+    joined = bufs.get_multi_cols(same_rows, dim=1).get_raw()
+    blocks = []
+    for k in same_rows:
+        b = -(-ref[k].shape[1] // world)
+        blocks.append(ref[k][:, rank * b : (rank + 1) * b])
+    assert torch.equal(joined.view(torch.int16), torch.cat(blocks, dim=1).view(torch.int16))
+    dims = OrderedDict((k, (-1 if v.dim() < 2 else i % 2)) for i, (k, v) in enumerate(ref.items()))
+    out = bufs.as_dict(dims)
+    for k, dim in dims.items():
+        want = ref[k]
+        if dim >= 0:
+            b = -(-want.shape[dim] // world)
+            want = want[(slice(None),) * dim + (slice(rank * b, (rank + 1) * b),)]
+        got = out[k].get_raw()
+        assert got.dtype == torch.bfloat16 and got.shape == want.shape, k
+        assert torch.equal(got.reshape(-1).view(torch.int16), want.reshape(-1).view(torch.int16)), k
+    del out, joined
+    bufs.close()
+    loader.close()
+    assert get_framework_op("pytorch").get_mem_used() == 0
 
 
 def test_loader_downcast_to_wider_type_is_refused(data_dir):
