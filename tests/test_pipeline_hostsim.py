@@ -176,6 +176,53 @@ def test_injected_read_fault(sim, blob):
     sim.fstx_ctx_destroy(ctx)
 
 
+def test_direct_reads_fail_cleanly(sim, blob, tmp_path):
+    """The same failures on the O_DIRECT path, where one read stages many blocks that other
+    workers ship: an injected read error, a failing device copy while staged blocks are in
+    flight, a file that ends early, and a destroy with staged work outstanding."""
+    path, data = blob
+    dev = np.zeros(data.size, dtype=np.uint8)
+    # injected read error: the second large read fails, every block of it reports -EIO
+    os.environ["FSTX_FAULT_READ_AFTER"] = "1"
+    try:
+        ctx = make_ctx(sim, block=64 * 1024, threads=4, direct_bytes=16 * 64 * 1024)
+    finally:
+        del os.environ["FSTX_FAULT_READ_AFTER"]
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_DIRECT)
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -5
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == data.size and np.array_equal(dev, data)
+    m = _native.FstxMetrics()
+    assert sim.fstx_get_metrics(ctx, ctypes.byref(m)) == 0
+    if m.direct_fallbacks == 0:  # the filesystem took O_DIRECT: the blocks went through the staged queue
+        assert m.blocks_direct > 0 and m.stage_ns > 0
+    # a failing device copy while staged blocks are being shipped
+    dev[:] = 0
+    sim.fstx_sim_fail_copy_after(7)
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -_native_code("HIP")
+    sim.fstx_sim_fail_copy_after(-1)
+    req = sim.fstx_submit_read(ctx, f, 4096, 1 << 20, dev.ctypes.data, dev.size, 4096)
+    assert sim.fstx_wait_read(ctx, req) == 1 << 20 and np.array_equal(dev[4096 : 4096 + (1 << 20)], data[4096 : 4096 + (1 << 20)])
+    # a file that ends inside a large read
+    cut = str(tmp_path / "cut.bin")
+    data[:600_000].tofile(cut)
+    g = sim.fstx_file_open(ctx, cut.encode(), _native.READ_DIRECT)
+    os.truncate(cut, 200_000)
+    req = sim.fstx_submit_read(ctx, g, 0, 600_000, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == -_native_code("SHORT_READ")
+    # destroy with direct requests outstanding: drains, leaves nothing behind
+    sim.fstx_sim_set_copy_delay_us(300)
+    dev[:] = 0
+    for k in range(3):
+        assert sim.fstx_submit_read(ctx, f, k * (1 << 20), 1 << 20, dev.ctypes.data, dev.size, k * (1 << 20)) >= 1
+    assert sim.fstx_ctx_destroy(ctx) == 0
+    sim.fstx_sim_set_copy_delay_us(30)
+    assert np.array_equal(dev[: 3 << 20], data[: 3 << 20])
+    assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+
+
 def test_destroy_with_requests_in_flight(sim, blob):
     path, data = blob
     sim.fstx_sim_set_copy_delay_us(300)
