@@ -339,3 +339,21 @@ def test_parallel_loader_error_and_early_stop(small_configs, tmp_path):
     it.close()
     del first
     assert_clean()
+
+
+def test_c_abi_from_plain_c(data_dir):
+    """A C99 program with no Python, torch or C++ in it loads a file through the pipeline
+    (three read modes, a destination range check) and runs the realign, slice, join and
+    convert entry points, checking every result against host loops."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi_native", "cabi_check.bin")
+    if not os.path.exists(exe):
+        pytest.skip("tests/cabi_native/cabi_check.bin is not built (run __graft_entry__.build())")
+    blob = os.path.join(data_dir, "cabi_blob.bin")
+    np.random.default_rng(3).integers(0, 256, 20_000_003, dtype=np.uint8).tofile(blob)
+    try:
+        run = subprocess.run([exe, blob], capture_output=True, text=True, timeout=120)
+    finally:
+        os.remove(blob)
+    assert run.returncode == 0 and "cabi_check: ok" in run.stdout, run.stdout + run.stderr
