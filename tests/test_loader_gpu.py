@@ -357,3 +357,38 @@ def test_c_abi_from_plain_c(data_dir):
     finally:
         os.remove(blob)
     assert run.returncode == 0 and "cabi_check: ok" in run.stdout, run.stdout + run.stderr
+
+
+def test_empty_tensors_and_files_without_data(tmp_path):
+    """Zero-element tensors between real ones, a file whose only tensor is empty, and a file
+    with no tensors at all load like any other (the reference's header rules allow them:
+    e - s == 0 == prod(shape) * itemsize, common.py:205-231)."""
+    from safetensors.torch import save_file
+
+    mixed = str(tmp_path / "mixed.safetensors")
+    save_file({"a": torch.arange(12, dtype=torch.float32).reshape(3, 4), "e": torch.empty((0, 7), dtype=torch.float16),
+               "z": torch.ones(5, dtype=torch.bfloat16), "e2": torch.empty(0, dtype=torch.int64)}, mixed)
+    only_empty = str(tmp_path / "only_empty.safetensors")
+    save_file({"only.e": torch.empty((4, 0), dtype=torch.float32)}, only_empty)
+    nothing = str(tmp_path / "nothing.safetensors")
+    save_file({}, nothing)
+    for layout in ("direct", "window"):
+        for rank, world in ((0, 1), (1, 2)):
+            pg = SingleGroup() if world == 1 else StubProcessGroup(rank, world)
+            loader = SafeTensorsFileLoader(pg, DEV, layout=layout, max_threads=2)
+            loader.add_filenames({rank: [mixed, only_empty, nothing]} if world > 1 else {0: [mixed, nothing]})
+            bufs = loader.copy_files_to_device()
+            bufs.auto_mem_delete = False
+            ref = load_file(mixed)
+            for k, t in ref.items():
+                got = bufs.get_tensor(k)
+                assert got.shape == t.shape and got.dtype == t.dtype and torch.equal(got.cpu(), t), (layout, k)
+                if world > 1 and t.dim() >= 1:
+                    sh = bufs.get_sharded(k, 0)
+                    b = -(-t.shape[0] // world)
+                    assert torch.equal(sh.cpu(), t[rank * b : (rank + 1) * b]), (layout, k)
+            if world > 1:
+                assert tuple(bufs.get_tensor("only.e").shape) == (4, 0)
+            bufs.close()
+            loader.close()
+            assert_clean()
