@@ -321,6 +321,35 @@ def test_join_copy_matches_cat(dev):
     assert lib.fstx_join_copy(a.data_ptr(), 0, 4, many, 25, None) == -10008
 
 
+def test_tensors_beyond_4_gib(dev):
+    """One tensor of 5.4 GB: byte offsets and unit indices past 2^32 in the realign copy
+    (shifted source), a column cut, a row cut and a conversion."""
+    rows, cols = 40960, 65536 + 8
+    t = torch.randint(-30000, 30000, (rows, cols), dtype=torch.int16, device=dev)
+    nbytes = t.numel() * 2
+    assert nbytes > 5 * (1 << 30)
+    flat = t.view(-1).view(torch.uint8)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    _native.realign_copy(out.data_ptr(), flat.data_ptr() + 6, nbytes - 6, stream())
+    assert torch.equal(out[: nbytes - 6], flat[6:])
+    assert torch.equal(out[nbytes - 4096 - 6 : nbytes - 6], flat[nbytes - 4096 :])
+    del out
+    half = cols // 2
+    cut = torch.empty((rows, half), dtype=torch.int16, device=dev)
+    _native.slice_copy(cut.data_ptr(), t.data_ptr() + half * 2, rows, half * 2, cols * 2, stream())
+    assert torch.equal(cut, t[:, half:])
+    del cut
+    block = rows // 2
+    rowcut = torch.empty((block, cols), dtype=torch.int16, device=dev)
+    _native.slice_copy(rowcut.data_ptr(), t.data_ptr() + block * cols * 2, 1, block * cols * 2, rows * cols * 2, stream())
+    assert torch.equal(rowcut, t[block:])
+    del rowcut, t
+    f = torch.randn(1_200_000_000, dtype=torch.float32, device=dev)  # 4.8 GB in, 2.4 GB out
+    o = torch.empty(f.numel(), dtype=torch.bfloat16, device=dev)
+    _native.convert_batch([(o.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], stream())
+    assert torch.equal(o.view(torch.int16), f.to(torch.bfloat16).view(torch.int16))
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
