@@ -344,6 +344,18 @@ def test_tensors_beyond_4_gib(dev):
     _native.slice_copy(rowcut.data_ptr(), t.data_ptr() + block * cols * 2, 1, block * cols * 2, rows * cols * 2, stream())
     assert torch.equal(rowcut, t[block:])
     del rowcut, t
+    # an odd column count: the LDS-staged kernel with more than 4 GiB per job (64-bit tile arithmetic)
+    rows, cols = 80000, 65537
+    t = torch.randint(-30000, 30000, (rows, cols), dtype=torch.int16, device=dev)
+    block = -(-cols // 2)
+    for rank in (0, 1):
+        width = min(block, cols - rank * block)
+        cut = torch.empty((rows, width), dtype=torch.int16, device=dev)
+        assert cut.numel() * 2 > (1 << 32)
+        _native.slice_copy(cut.data_ptr(), t.data_ptr() + rank * block * 2, rows, width * 2, cols * 2, stream())
+        assert torch.equal(cut, t[:, rank * block : rank * block + width]), rank
+        del cut
+    del t
     f = torch.randn(1_200_000_000, dtype=torch.float32, device=dev)  # 4.8 GB in, 2.4 GB out
     o = torch.empty(f.numel(), dtype=torch.bfloat16, device=dev)
     _native.convert_batch([(o.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], stream())
