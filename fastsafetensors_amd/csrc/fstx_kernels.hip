@@ -725,8 +725,13 @@ inline uint32_t common_unit_log2(uint64_t bits) {
     return l;
 }
 
-constexpr uint64_t kMaxUnitsPerJob = 0xffffff00ull; // keeps lb * 256 + lane in 32 bits
-constexpr uint64_t kMaxBlocksPerLaunch = 0x3fffff00ull; // leaves room for granule padding
+// The size of a launch is counted in work-items with 32 bits: at most 2^32 - 1 lanes, 67.1 M
+// workgroups of 64.  Launches are planned up to 56 M workgroups, which leaves room for the
+// idle workgroups that pad jobs to granules and eighths; one job takes at most 48 M.
+constexpr uint64_t kMaxBlocksPerLaunch = 56ull << 20;
+constexpr uint64_t kMaxBlocksPerJob = 48ull << 20;
+constexpr uint64_t kMaxUnitsPerJob = kMaxBlocksPerJob * kBlock; // 3.2 G: unit indices stay in 32 bits
+inline bool grid_fits(uint64_t workgroups) { return workgroups * kBlock <= 0xffffffffull; }
 
 } // namespace
 
@@ -738,6 +743,20 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
     uint64_t blocks_of[FSTX_BATCH_MAX];
     uint64_t sum = 0;
     uint32_t k = 0;
+    auto flush = [&]() -> int {
+        if (k == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t blocks = plan_grid(t, blocks_of, k, &gl);
+        if (!grid_fits(blocks)) return -FSTX_E_RANGE;
+        hipLaunchKernelGGL(realign_kernel, dim3((uint32_t)blocks), dim3(kBlock), 0,
+                           static_cast<hipStream_t>(stream), gl, t);
+        k = 0;
+        sum = 0;
+        return fstx_internal::check_launch("realign_kernel");
+    };
+    // a span larger than one job may be is cut into pieces (any multiple of 16 bytes keeps
+    // the relative alignment of source and destination)
+    const uint64_t piece = kMaxBlocksPerJob * (uint64_t)kBlock * kVecBytes;
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_copy_desc &d = descs[i];
         if (d.nbytes == 0) continue;
@@ -745,32 +764,25 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
         const char *s = static_cast<const char *>(d.src);
         char *o = static_cast<char *>(d.dst);
         if ((s < o + d.nbytes) && (o < s + d.nbytes)) return -FSTX_E_INVAL; // overlap
-        t.job[k] = RealignJob{o, s, d.nbytes, 0};
-        blocks_of[k] = (blocks_for(d.nbytes / kVecBytes) + kXcds - 1) / kXcds * kXcds;
-        sum += blocks_of[k];
-        if (sum > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
-        ++k;
+        for (uint64_t done = 0; done < d.nbytes; done += piece) {
+            const uint64_t len = d.nbytes - done < piece ? d.nbytes - done : piece;
+            const uint64_t need = (blocks_for(len / kVecBytes) + kXcds - 1) / kXcds * kXcds;
+            if (k == FSTX_BATCH_MAX || sum + need > kMaxBlocksPerLaunch) {
+                int rc = flush();
+                if (rc < 0) return rc;
+            }
+            t.job[k] = RealignJob{o + done, s + done, len, 0};
+            blocks_of[k] = need;
+            sum += need;
+            ++k;
+        }
     }
-    if (k == 0) return 0;
-    uint32_t gl = 0;
-    const uint64_t blocks = plan_grid(t, blocks_of, k, &gl);
-    hipLaunchKernelGGL(realign_kernel, dim3((uint32_t)blocks), dim3(kBlock), 0,
-                       static_cast<hipStream_t>(stream), gl, t);
-    return fstx_internal::check_launch("realign_kernel");
+    return flush();
 }
 
 extern "C" int fstx_realign_copy(void *dst, const void *src, uint64_t nbytes, void *stream) {
-    // one launch covers < 2^31 workgroups of 4 KiB; split beyond that
-    const uint64_t piece = (kMaxBlocksPerLaunch - 1) * (uint64_t)kBlock * kVecBytes;
-    uint64_t done = 0;
-    do {
-        uint64_t len = nbytes - done < piece ? nbytes - done : piece;
-        fstx_copy_desc d{static_cast<char *>(dst) + done, static_cast<const char *>(src) + done, len};
-        int rc = fstx_realign_copy_batch(&d, 1, stream);
-        if (rc < 0) return rc;
-        done += len;
-    } while (done < nbytes);
-    return 0;
+    fstx_copy_desc d{dst, src, nbytes};
+    return fstx_realign_copy_batch(&d, 1, stream);
 }
 
 extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, void *stream) {
@@ -786,6 +798,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         if (kl == 0) return 0;
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(tl, tiles_of, kl, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
         hipLaunchKernelGGL(slice_lds_kernel, dim3((uint32_t)grid), dim3(64), lds_bytes_for(min_seg),
                            static_cast<hipStream_t>(stream), gl, tl);
         kl = 0;
@@ -797,6 +810,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         if (k == 0) return 0;
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
         hipLaunchKernelGGL(slice_kernel, dim3((uint32_t)grid), dim3(kBlock), 0,
                            static_cast<hipStream_t>(stream), gl, t);
         k = 0;
@@ -820,7 +834,8 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src |
                                              seg | pitch | 16u);
         if (ul < 4 && seg >= kLdsMinSeg && seg < 0x80000000ull && outer <= 0xffffffffull &&
-            ((uintptr_t)d.dst & 15) == 0 && !fstx_internal::lds_path_disabled()) {
+            ((uintptr_t)d.dst & 15) == 0 && (outer * seg + kTileBytes - 1) / kTileBytes + kXcds <= kMaxBlocksPerJob &&
+            !fstx_internal::lds_path_disabled()) {
             // odd alignment somewhere: keep the global accesses 16 bytes wide and realign through LDS
             const uint64_t n_tiles = (outer * seg + kTileBytes - 1) / kTileBytes;
             if (kl == FSTX_BATCH_MAX || tiles + n_tiles + kXcds > kMaxBlocksPerLaunch) {
@@ -838,7 +853,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         const uint64_t seg_units = seg >> ul;
         // rows per job so that the unit index fits 32 bits
         uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
-        if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 4 Gi units or more
+        if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more
         for (uint64_t row = 0; row < outer; row += rows_per_job) {
             uint64_t rows = outer - row < rows_per_job ? outer - row : rows_per_job;
             uint64_t units = rows * seg_units;
@@ -879,6 +894,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         if (k == 0) return 0;
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
         hipLaunchKernelGGL(slice2d_kernel, dim3((uint32_t)grid), dim3(kBlock), 0,
                            static_cast<hipStream_t>(stream), gl, t);
         k = 0;
@@ -901,7 +917,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
                                              d.src_pitch | d.dst_pitch | 16u);
         const uint64_t seg_units = d.seg_bytes >> ul;
         uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
-        if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 4 Gi units or more
+        if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more
         for (uint64_t row = 0; row < d.outer; row += rows_per_job) {
             const uint64_t rows = d.outer - row < rows_per_job ? d.outer - row : rows_per_job;
             const uint64_t units = rows * seg_units;
@@ -963,12 +979,23 @@ extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, cons
         col += s.seg_bytes;
         ++t.n;
     }
-    const uint64_t chunks = (rows + rpc - 1) / rpc;
-    if (waves > 0xffffffffull || chunks * waves > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
+    if (waves == 0 || waves > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
     t.waves_per_chunk = (uint32_t)waves;
-    hipLaunchKernelGGL(join_kernel, dim3((uint32_t)(chunks * waves)), dim3(kBlock), 0,
-                       static_cast<hipStream_t>(stream), t);
-    return fstx_internal::check_launch("join_kernel");
+    // as many chunks per launch as the grid allows; the next launch continues further down
+    const uint64_t chunks_per_launch = kMaxBlocksPerLaunch / waves;
+    for (uint64_t row = 0; row < rows; row += chunks_per_launch * rpc) {
+        const uint64_t part = rows - row < chunks_per_launch * rpc ? rows - row : chunks_per_launch * rpc;
+        JoinTable tt = t;
+        tt.dst += row * dst_pitch;
+        tt.rows = (uint32_t)part;
+        for (uint32_t j = 0; j < tt.n; ++j) tt.src[j].src += row * tt.src[j].src_pitch;
+        const uint64_t grid = (part + rpc - 1) / rpc * waves;
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        hipLaunchKernelGGL(join_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream), tt);
+        int rc = fstx_internal::check_launch("join_kernel");
+        if (rc < 0) return rc;
+    }
+    return 0;
 }
 
 extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {
@@ -980,6 +1007,17 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
     uint64_t blocks_of[FSTX_BATCH_MAX];
     uint64_t sum = 0;
     uint32_t k = 0;
+    auto flush = [&]() -> int {
+        if (k == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        hipLaunchKernelGGL(convert_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                           gl, t);
+        k = 0;
+        sum = 0;
+        return fstx_internal::check_launch("convert_kernel");
+    };
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_convert_desc &d = descs[i];
         if (d.n_elems == 0) continue;
@@ -991,17 +1029,20 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         const char *sb = static_cast<const char *>(d.src);
         char *db = static_cast<char *>(d.dst);
         if (sb < db + d.n_elems * ds && db < sb + d.n_elems * ss) return -FSTX_E_INVAL; // overlap
-        t.job[k] = ConvertJob{db, sb, d.n_elems, d.src_type, d.dst_type};
         const uint64_t per_block = (uint64_t)kBlock * (16 / ss);
-        blocks_of[k] = (d.n_elems + per_block - 1) / per_block;
-        sum += blocks_of[k];
-        if (sum > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
-        ++k;
+        const uint64_t piece = kMaxBlocksPerJob * per_block; // elements one job may take
+        for (uint64_t done = 0; done < d.n_elems; done += piece) {
+            const uint64_t len = d.n_elems - done < piece ? d.n_elems - done : piece;
+            const uint64_t need = (len + per_block - 1) / per_block;
+            if (k == FSTX_BATCH_MAX || sum + need > kMaxBlocksPerLaunch) {
+                int rc = flush();
+                if (rc < 0) return rc;
+            }
+            t.job[k] = ConvertJob{db + done * ds, sb + done * ss, len, d.src_type, d.dst_type};
+            blocks_of[k] = need;
+            sum += need;
+            ++k;
+        }
     }
-    if (k == 0) return 0;
-    uint32_t gl = 0;
-    const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
-    hipLaunchKernelGGL(convert_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
-                       gl, t);
-    return fstx_internal::check_launch("convert_kernel");
+    return flush();
 }

@@ -356,6 +356,35 @@ def test_tensors_beyond_4_gib(dev):
         assert torch.equal(cut, t[:, rank * block : rank * block + width]), rank
         del cut
     del t
+    # one-byte units (odd pitch): more than 2^32 units, so the direct kernels split the tensor
+    # into several jobs by rows
+    import os
+
+    rows, cols = 80000, 65537
+    t = torch.randint(0, 255, (rows, cols), dtype=torch.uint8, device=dev)
+    cut = torch.empty((rows, cols - 1), dtype=torch.uint8, device=dev)
+    os.environ["FSTX_NO_LDS_SLICE"] = "1"
+    try:
+        _native.slice_copy(cut.data_ptr(), t.data_ptr(), rows, cols - 1, cols, stream())
+    finally:
+        os.environ.pop("FSTX_NO_LDS_SLICE")
+    assert torch.equal(cut, t[:, :-1])
+    cut.zero_()
+    wide = torch.zeros((rows, cols + 2), dtype=torch.uint8, device=dev)
+    _native.slice_copy2d_batch([(wide.data_ptr() + 1, t.data_ptr(), rows, cols - 1, cols, cols + 2)], stream())
+    assert torch.equal(wide[:, 1:cols], t[:, :-1]) and not wide[:, 0].any() and not wide[:, cols:].any()
+    del t, cut, wide
+    # a span of 56 GiB: more than one job, and more than one launch, may cover
+    n = (56 << 30) + 12345
+    big = torch.empty(n + 64, dtype=torch.uint8, device=dev)
+    for at in range(0, n + 64, 1 << 32):
+        big[at : at + (1 << 32)].random_(0, 255)
+    out = torch.empty(n, dtype=torch.uint8, device=dev)
+    _native.realign_copy(out.data_ptr(), big.data_ptr() + 3, n, stream())
+    assert torch.equal(out, big[3 : 3 + n])
+    _native.realign_copy_batch([(out.data_ptr(), big.data_ptr() + 16, n), (big.data_ptr() + n + 32, big.data_ptr(), 32)], stream())
+    assert torch.equal(out, big[16 : 16 + n]) and torch.equal(big[n + 32 : n + 64], big[:32])
+    del big, out
     f = torch.randn(1_200_000_000, dtype=torch.float32, device=dev)  # 4.8 GB in, 2.4 GB out
     o = torch.empty(f.numel(), dtype=torch.bfloat16, device=dev)
     _native.convert_batch([(o.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], stream())
