@@ -24,6 +24,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "fstx.h"
 #include "fstx_internal.h"
@@ -728,9 +729,19 @@ inline uint32_t common_unit_log2(uint64_t bits) {
 // The size of a launch is counted in work-items with 32 bits: at most 2^32 - 1 lanes, 67.1 M
 // workgroups of 64.  Launches are planned up to 56 M workgroups, which leaves room for the
 // idle workgroups that pad jobs to granules and eighths; one job takes at most 48 M.
-constexpr uint64_t kMaxBlocksPerLaunch = 56ull << 20;
-constexpr uint64_t kMaxBlocksPerJob = 48ull << 20;
-constexpr uint64_t kMaxUnitsPerJob = kMaxBlocksPerJob * kBlock; // 3.2 G: unit indices stay in 32 bits
+struct Limits {
+    uint64_t launch; // workgroups one launch is planned up to
+    uint64_t job;    // workgroups one job may take
+    uint64_t units() const { return job * kBlock; } // 3.2 G at most: unit indices stay in 32 bits
+};
+// FSTX_MAX_BLOCKS_PER_LAUNCH shrinks the limits so that tests reach the cutting logic with small tensors.
+inline Limits limits() {
+    if (const char *e = getenv("FSTX_MAX_BLOCKS_PER_LAUNCH")) {
+        const uint64_t v = strtoull(e, nullptr, 10);
+        if (v >= 64 && v <= (56ull << 20)) return Limits{v, v - v / 8};
+    }
+    return Limits{56ull << 20, 48ull << 20};
+}
 inline bool grid_fits(uint64_t workgroups) { return workgroups * kBlock <= 0xffffffffull; }
 
 } // namespace
@@ -756,7 +767,8 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
     };
     // a span larger than one job may be is cut into pieces (any multiple of 16 bytes keeps
     // the relative alignment of source and destination)
-    const uint64_t piece = kMaxBlocksPerJob * (uint64_t)kBlock * kVecBytes;
+    const Limits lim = limits();
+    const uint64_t piece = lim.job * (uint64_t)kBlock * kVecBytes;
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_copy_desc &d = descs[i];
         if (d.nbytes == 0) continue;
@@ -767,7 +779,7 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
         for (uint64_t done = 0; done < d.nbytes; done += piece) {
             const uint64_t len = d.nbytes - done < piece ? d.nbytes - done : piece;
             const uint64_t need = (blocks_for(len / kVecBytes) + kXcds - 1) / kXcds * kXcds;
-            if (k == FSTX_BATCH_MAX || sum + need > kMaxBlocksPerLaunch) {
+            if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
@@ -819,6 +831,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     };
     fstx_copy_desc spans[FSTX_BATCH_MAX];
     uint32_t n_spans = 0;
+    const Limits lim = limits();
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_slice_desc &d = descs[i];
         if (d.outer == 0 || d.seg_bytes == 0) continue;
@@ -834,11 +847,11 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src |
                                              seg | pitch | 16u);
         if (ul < 4 && seg >= kLdsMinSeg && seg < 0x80000000ull && outer <= 0xffffffffull &&
-            ((uintptr_t)d.dst & 15) == 0 && (outer * seg + kTileBytes - 1) / kTileBytes + kXcds <= kMaxBlocksPerJob &&
+            ((uintptr_t)d.dst & 15) == 0 && (outer * seg + kTileBytes - 1) / kTileBytes + kXcds <= lim.job &&
             !fstx_internal::lds_path_disabled()) {
             // odd alignment somewhere: keep the global accesses 16 bytes wide and realign through LDS
             const uint64_t n_tiles = (outer * seg + kTileBytes - 1) / kTileBytes;
-            if (kl == FSTX_BATCH_MAX || tiles + n_tiles + kXcds > kMaxBlocksPerLaunch) {
+            if (kl == FSTX_BATCH_MAX || tiles + n_tiles + kXcds > lim.launch) {
                 int rc = flush_lds();
                 if (rc < 0) return rc;
             }
@@ -852,12 +865,12 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         }
         const uint64_t seg_units = seg >> ul;
         // rows per job so that the unit index fits 32 bits
-        uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
+        uint64_t rows_per_job = lim.units() / seg_units;
         if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more
         for (uint64_t row = 0; row < outer; row += rows_per_job) {
             uint64_t rows = outer - row < rows_per_job ? outer - row : rows_per_job;
             uint64_t units = rows * seg_units;
-            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > kMaxBlocksPerLaunch) {
+            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
@@ -903,6 +916,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
     };
     fstx_slice_desc dense[FSTX_BATCH_MAX];
     uint32_t n_dense = 0;
+    const Limits lim = limits();
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_slice2d_desc &d = descs[i];
         if (d.outer == 0 || d.seg_bytes == 0) continue;
@@ -916,12 +930,12 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
                                              d.src_pitch | d.dst_pitch | 16u);
         const uint64_t seg_units = d.seg_bytes >> ul;
-        uint64_t rows_per_job = kMaxUnitsPerJob / seg_units;
+        uint64_t rows_per_job = lim.units() / seg_units;
         if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more
         for (uint64_t row = 0; row < d.outer; row += rows_per_job) {
             const uint64_t rows = d.outer - row < rows_per_job ? d.outer - row : rows_per_job;
             const uint64_t units = rows * seg_units;
-            if (k == kJobs || blocks + blocks_for(units) > kMaxBlocksPerLaunch) {
+            if (k == kJobs || blocks + blocks_for(units) > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
@@ -966,23 +980,32 @@ extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, cons
     // lanes at the end of each source's share of a chunk stay below a few percent
     uint64_t rpc = (16ull * kBlock + (min_seg >> ul) - 1) / (min_seg >> ul);
     if (rpc > rows) rpc = rows;
+    const Limits lim = limits();
+    auto waves_of = [&](uint64_t rows_per_chunk) {
+        uint64_t w = 0;
+        for (uint32_t i = 0; i < n; ++i)
+            w += (rows_per_chunk * (srcs[i].seg_bytes >> ul) + kBlock - 1) / kBlock;
+        return w;
+    };
+    // ... unless a very short block next to very long ones would make one chunk larger than a launch
+    while (rpc > 1 && (waves_of(rpc) > lim.launch || rpc * (row_bytes >> ul) > lim.units())) rpc /= 2;
     t.rows_per_chunk = (uint32_t)rpc;
     uint64_t waves = 0, col = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_join_src &s = srcs[i];
         if (s.seg_bytes == 0) continue;
         const uint64_t units = rpc * (s.seg_bytes >> ul);
-        if (units > kMaxUnitsPerJob) return -FSTX_E_RANGE;
+        if (units > lim.units()) return -FSTX_E_RANGE;
         t.wave_begin[t.n] = (uint32_t)waves;
         t.src[t.n] = JoinSrc{static_cast<const char *>(s.src), s.src_pitch, (uint32_t)(s.seg_bytes >> ul), (uint32_t)col, 0};
         waves += (units + kBlock - 1) / kBlock;
         col += s.seg_bytes;
         ++t.n;
     }
-    if (waves == 0 || waves > kMaxBlocksPerLaunch) return -FSTX_E_RANGE;
+    if (waves == 0 || waves > lim.launch) return -FSTX_E_RANGE; // one joined row is more than a launch holds
     t.waves_per_chunk = (uint32_t)waves;
     // as many chunks per launch as the grid allows; the next launch continues further down
-    const uint64_t chunks_per_launch = kMaxBlocksPerLaunch / waves;
+    const uint64_t chunks_per_launch = lim.launch / waves;
     for (uint64_t row = 0; row < rows; row += chunks_per_launch * rpc) {
         const uint64_t part = rows - row < chunks_per_launch * rpc ? rows - row : chunks_per_launch * rpc;
         JoinTable tt = t;
@@ -1003,6 +1026,7 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
     if (!descs) return -FSTX_E_INVAL;
     if (n > FSTX_BATCH_MAX) return -FSTX_E_TOO_MANY;
     static const uint32_t size_of[6] = {8, 4, 2, 2, 1, 1};
+    const Limits lim = limits();
     JobTable<ConvertJob> t;
     uint64_t blocks_of[FSTX_BATCH_MAX];
     uint64_t sum = 0;
@@ -1030,11 +1054,11 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         char *db = static_cast<char *>(d.dst);
         if (sb < db + d.n_elems * ds && db < sb + d.n_elems * ss) return -FSTX_E_INVAL; // overlap
         const uint64_t per_block = (uint64_t)kBlock * (16 / ss);
-        const uint64_t piece = kMaxBlocksPerJob * per_block; // elements one job may take
+        const uint64_t piece = lim.job * per_block; // elements one job may take
         for (uint64_t done = 0; done < d.n_elems; done += piece) {
             const uint64_t len = d.n_elems - done < piece ? d.n_elems - done : piece;
             const uint64_t need = (len + per_block - 1) / per_block;
-            if (k == FSTX_BATCH_MAX || sum + need > kMaxBlocksPerLaunch) {
+            if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }

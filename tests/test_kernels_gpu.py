@@ -391,6 +391,34 @@ def test_tensors_beyond_4_gib(dev):
     assert torch.equal(o.view(torch.int16), f.to(torch.bfloat16).view(torch.int16))
 
 
+def test_cutting_into_jobs_and_launches(dev, monkeypatch):
+    """With the launch limits shrunk to a few thousand workgroups the same random sweeps go
+    through the code that cuts spans, tensors and joins into several jobs and launches."""
+    monkeypatch.setenv("FSTX_MAX_BLOCKS_PER_LAUNCH", "4096")
+    test_realign_batch_many_jobs(dev)
+    test_slice_odd_shapes_go_through_lds(dev)
+    test_slice_lds_random_geometry_in_one_batch(dev)
+    test_slice2d_strided_destination(dev)
+    test_join_copy_matches_cat(dev)
+    # one span, one strided tensor, one join and one conversion that are each many launches long
+    n = 40_000_003
+    src = torch.randint(0, 255, (n + 16,), dtype=torch.uint8, device=dev)
+    out = torch.zeros(n + 16, dtype=torch.uint8, device=dev)
+    _native.realign_copy(out.data_ptr(), src.data_ptr() + 5, n, stream())
+    assert torch.equal(out[:n], src[5 : 5 + n]) and not out[n:].any()
+    t = src[: 6000 * 6000].view(6000, 6000)
+    cut = torch.empty((6000, 3000), dtype=torch.uint8, device=dev)
+    _native.slice_copy(cut.data_ptr(), t.data_ptr() + 3000, 6000, 3000, 6000, stream())
+    assert torch.equal(cut, t[:, 3000:])
+    joined = torch.empty((6000, 4500), dtype=torch.uint8, device=dev)
+    _native.join_copy(joined.data_ptr(), 6000, [(t.data_ptr(), 3000, 6000), (t.data_ptr() + 4000, 1500, 6000)], stream())
+    assert torch.equal(joined, torch.cat([t[:, :3000], t[:, 4000:5500]], dim=1))
+    f = torch.randn(9_000_001, dtype=torch.float32, device=dev)
+    o = torch.zeros(f.numel() + 8, dtype=torch.bfloat16, device=dev)
+    _native.convert_batch([(o.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], stream())
+    assert torch.equal(o[: f.numel()].view(torch.int16), f.to(torch.bfloat16).view(torch.int16)) and not o[f.numel() :].view(torch.int16).any()
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
