@@ -419,6 +419,57 @@ def test_cutting_into_jobs_and_launches(dev, monkeypatch):
     assert torch.equal(o[: f.numel()].view(torch.int16), f.to(torch.bfloat16).view(torch.int16)) and not o[f.numel() :].view(torch.int16).any()
 
 
+def test_entry_points_can_be_captured_in_a_graph(dev):
+    """The kernel entry points only enqueue work (no allocation, no synchronisation, tables
+    passed by value), so a caller may record them into a HIP graph: three replays, each after
+    the sources were changed by eager work, each compared with an eager run."""
+    rows, cols = 512, 4096
+    a = torch.randint(-3000, 3000, (rows, cols), dtype=torch.int16, device=dev)
+    b = torch.randint(-3000, 3000, (rows, cols + 6), dtype=torch.int16, device=dev)  # odd pitch: LDS kernel
+    f = torch.randn(rows * cols, dtype=torch.float32, device=dev)
+    cut_a = torch.empty((rows, cols // 4), dtype=torch.int16, device=dev)
+    cut_b = torch.empty((rows, 1001), dtype=torch.int16, device=dev)
+    moved = torch.empty(rows * cols * 2 - 6, dtype=torch.uint8, device=dev)
+    joined = torch.empty((rows, cols // 4 + 1001), dtype=torch.int16, device=dev)
+    half = torch.empty(rows * cols, dtype=torch.bfloat16, device=dev)
+
+    def enqueue(st):
+        _native.slice_copy_batch([(cut_a.data_ptr(), a.data_ptr() + cols // 4 * 2, rows, cols // 4 * 2, cols * 2),
+                                  (cut_b.data_ptr(), b.data_ptr() + 6, rows, 1001 * 2, (cols + 6) * 2)], st)
+        _native.realign_copy(moved.data_ptr(), a.data_ptr() + 6, moved.numel(), st)
+        _native.join_copy(joined.data_ptr(), rows, [(a.data_ptr() + cols // 4 * 2, cols // 4 * 2, cols * 2),
+                                                    (b.data_ptr() + 6, 1001 * 2, (cols + 6) * 2)], st)
+        _native.convert_batch([(half.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], st)
+
+    def check():
+        assert torch.equal(cut_a, a[:, cols // 4 : cols // 2])
+        assert torch.equal(cut_b, b[:, 3 : 3 + 1001])
+        assert torch.equal(moved, a.view(-1).view(torch.uint8)[6:])
+        assert torch.equal(joined, torch.cat([a[:, cols // 4 : cols // 2], b[:, 3 : 3 + 1001]], dim=1))
+        assert torch.equal(half.view(torch.int16), f.to(torch.bfloat16).view(torch.int16))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue(side.cuda_stream)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue(torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        a.add_(replay + 1)  # eager work between the replays
+        b.mul_(-1)
+        f.mul_(1.5)
+        for t in (cut_a, cut_b, moved, joined):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check()
+
+
 def test_slice_zero_sized_and_errors(dev):
     a = torch.zeros(4096, dtype=torch.uint8, device=dev)
     _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 0, 16, 32, stream())  # nothing to do
