@@ -52,47 +52,20 @@ class Device:
         return self.type is not DeviceType.CPU
 
 
-class DType(Enum):
-    BOOL = "BOOL"
-    I8 = "I8"
-    I16 = "I16"
-    I32 = "I32"
-    I64 = "I64"
-    U8 = "U8"
-    U16 = "U16"
-    U32 = "U32"
-    U64 = "U64"
-    F16 = "F16"
-    F32 = "F32"
-    F64 = "F64"
-    BF16 = "BF16"
-    F8_E5M2 = "F8_E5M2"
-    F8_E4M3 = "F8_E4M3"
-    F8_E8M0 = "F8_E8M0"
-    F4 = "F4"
-    AUTO = "AUTO"
-
-
-# bits per logical element; F4 packs two values per byte
-_DTYPE_BITS = {
-    DType.BOOL: 8,
-    DType.I8: 8,
-    DType.U8: 8,
-    DType.F8_E5M2: 8,
-    DType.F8_E4M3: 8,
-    DType.F8_E8M0: 8,
-    DType.F4: 4,
-    DType.I16: 16,
-    DType.U16: 16,
-    DType.F16: 16,
-    DType.BF16: 16,
-    DType.I32: 32,
-    DType.U32: 32,
-    DType.F32: 32,
-    DType.I64: 64,
-    DType.U64: 64,
-    DType.F64: 64,
+# safetensors dtype tag -> bits per logical element (F4 packs two values per byte)
+_TAG_BITS = {
+    "BOOL": 8, "I8": 8, "U8": 8, "F8_E5M2": 8, "F8_E4M3": 8, "F8_E8M0": 8, "F4": 4,
+    "I16": 16, "U16": 16, "F16": 16, "BF16": 16,
+    "I32": 32, "U32": 32, "F32": 32,
+    "I64": 64, "U64": 64, "F64": 64,
 }
+
+# One member per tag, valued by the tag itself (``DType("BF16") is DType.BF16``), plus AUTO
+# for "as stored in the file".  Same names as ``st_types.py:45-63`` of the reference.
+DType = Enum("DType", {tag: tag for tag in (*_TAG_BITS, "AUTO")}, module=__name__)
+DType.__doc__ = "Element type tag of a safetensors header; AUTO means: as stored."
+
+_DTYPE_BITS = {DType(tag): bits for tag, bits in _TAG_BITS.items()}
 
 
 def dtype_bits(dtype: DType) -> int:
