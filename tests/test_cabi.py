@@ -110,3 +110,28 @@ def test_without_a_gpu_the_product_refuses_loudly():
         SafeTensorsFileLoader(SingleGroup(), "cuda:0")  # and no silent fallback either
     with pytest.raises(_native.NativeError, match="no HIP device"):
         _native.Reader(0)
+
+
+def test_the_product_never_reaches_for_the_oracle_or_scratch_files():
+    """The oracle is test infrastructure: nothing under fastsafetensors_amd/ may import it
+    (or anything from the builder's scratch directory), and bench.py may only inside its
+    CPU baseline."""
+    import ast
+    import glob
+
+    def imported(path):
+        mods = set()
+        for node in ast.walk(ast.parse(open(path).read())):
+            if isinstance(node, ast.Import):
+                mods |= {a.name.split(".")[0] for a in node.names}
+            elif isinstance(node, ast.ImportFrom) and node.module and node.level == 0:
+                mods.add(node.module.split(".")[0])
+        return mods
+
+    for path in glob.glob(os.path.join(ROOT, "fastsafetensors_amd", "**", "*.py"), recursive=True):
+        assert not imported(path) & {"oracle", "_work"}, path
+    tree = ast.parse(open(os.path.join(ROOT, "bench.py")).read())
+    for fn in [n for n in tree.body if isinstance(n, ast.FunctionDef)]:
+        uses = any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in ast.walk(fn))
+        assert uses == (fn.name == "cpu_baseline"), fn.name
+    assert not any(isinstance(n, (ast.Import, ast.ImportFrom)) and "oracle" in ast.dump(n) for n in tree.body)
