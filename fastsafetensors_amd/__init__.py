@@ -3,6 +3,7 @@
 
 __version__ = "0.1.0"
 
+from .copier.mi355x import hold_reader
 from .common import SafeTensorsMetadata, SingleGroup, TensorFrame, get_device_numa_node
 from .file_buffer import FilesBufferOnDevice
 from .frameworks._torch import StubProcessGroup
@@ -25,4 +26,5 @@ __all__ = [
     "TensorFrame",
     "fastsafe_open",
     "get_device_numa_node",
+    "hold_reader",
 ]

@@ -17,10 +17,11 @@ _LIB_NAME = "libfstx.so"
 _lib: Optional[ctypes.CDLL] = None
 _lib_lock = threading.Lock()
 
-FSTX_ABI_VERSION = 1
+FSTX_ABI_VERSION = 2
 FSTX_BATCH_MAX = 48
 READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
 ADAPTIVE_DEPTH = 1
+PROBE_NO_COPY, PROBE_NO_READ = 2, 4
 READ_MODES = {"auto": READ_AUTO, "buffered": READ_BUFFERED, "direct": READ_DIRECT}
 
 
@@ -44,7 +45,7 @@ class FstxConfig(ctypes.Structure):
         ("max_direct_reads", ctypes.c_uint32),
         ("direct_read_bytes", ctypes.c_uint64),
         ("flags", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32),
+        ("direct_ramp_kb", ctypes.c_uint32),
     ]
 
 
@@ -62,6 +63,8 @@ class FstxMetrics(ctypes.Structure):
             "slot_wait_ns",
             "direct_fallbacks",
             "direct_depth",
+            "direct_reads",
+            "create_ns",
         )
     ]
 
@@ -106,6 +109,16 @@ class FstxConvertDesc(ctypes.Structure):
 
 
 ELEM_TYPES = {"F64": 0, "F32": 1, "F16": 2, "BF16": 3, "F8_E4M3": 4, "F8_E5M2": 5}
+_ELEM_BYTES = {"F64": 8, "F32": 4, "F16": 2, "BF16": 2, "F8_E4M3": 1, "F8_E5M2": 1}
+
+
+def convert_supported(src: str, dst: str) -> bool:
+    """Whether ``fstx_convert_batch`` has a kernel for this pair of safetensors dtype tags:
+    from f64 / f32 / f16 / bf16 towards a different float type that is not wider."""
+    return (
+        src in ELEM_TYPES and dst in ELEM_TYPES and src != dst and not src.startswith("F8")
+        and dst != "F64" and _ELEM_BYTES[dst] <= _ELEM_BYTES[src]
+    )
 
 # name -> (restype, argtypes); must list every function include/fstx.h declares
 _SIGNATURES = {
@@ -121,6 +134,9 @@ _SIGNATURES = {
     "fstx_host_free": (None, [ctypes.c_void_p]),
     "fstx_ctx_create": (ctypes.c_int, [ctypes.POINTER(FstxConfig), ctypes.POINTER(ctypes.c_void_p)]),
     "fstx_ctx_destroy": (ctypes.c_int, [ctypes.c_void_p]),
+    "fstx_ctx_acquire": (ctypes.c_int, [ctypes.POINTER(FstxConfig), ctypes.POINTER(ctypes.c_void_p)]),
+    "fstx_ctx_release": (ctypes.c_int, [ctypes.c_void_p]),
+    "fstx_ctx_order_after": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "fstx_file_open": (ctypes.c_int64, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int]),
     "fstx_file_close": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64]),
     "fstx_submit_read": (
@@ -354,7 +370,13 @@ def convert_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 
 
 
 class Reader:
-    """One copy pipeline: worker threads, pinned ring and copy streams."""
+    """One copy pipeline: worker threads, pinned ring and copy streams.
+
+    ``shared=True`` asks the library for the process-wide context of this configuration
+    (``fstx_ctx_acquire``): readers that are alive at the same time then use one set of
+    threads, one ring and one set of streams, and the last ``close`` frees them.
+    ``probe`` is ``PROBE_NO_COPY`` or ``PROBE_NO_READ`` for a measurement context.
+    """
 
     def __init__(
         self,
@@ -367,13 +389,21 @@ class Reader:
         max_direct_reads: int = 0,
         direct_read_bytes: int = 0,
         adaptive_depth: bool = False,
+        direct_ramp_kb: int = 0,
+        probe: int = 0,
+        shared: bool = False,
     ):
         cfg = FstxConfig(
             ctypes.sizeof(FstxConfig), device_id, numa_node, n_threads, n_streams, block_bytes,
-            slots_per_thread, max_direct_reads, direct_read_bytes, ADAPTIVE_DEPTH if adaptive_depth else 0, 0,
+            slots_per_thread, max_direct_reads, direct_read_bytes,
+            (ADAPTIVE_DEPTH if adaptive_depth else 0) | probe, direct_ramp_kb,
         )
         handle = ctypes.c_void_p()
-        _check("fstx_ctx_create", lib().fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(handle)))
+        self._shared = shared
+        if shared:
+            _check("fstx_ctx_acquire", lib().fstx_ctx_acquire(ctypes.byref(cfg), ctypes.byref(handle)))
+        else:
+            _check("fstx_ctx_create", lib().fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(handle)))
         self._ctx: Optional[ctypes.c_void_p] = handle
 
     def _h(self) -> ctypes.c_void_p:
@@ -403,10 +433,14 @@ class Reader:
         _check("fstx_get_metrics", lib().fstx_get_metrics(self._h(), ctypes.byref(m)))
         return m
 
+    def order_after(self, stream: int) -> None:
+        """Copies of requests submitted from now on start after the work queued on ``stream``."""
+        _check("fstx_ctx_order_after", lib().fstx_ctx_order_after(self._h(), stream))
+
     def close(self) -> None:
         if self._ctx is not None:
             ctx, self._ctx = self._ctx, None
-            lib().fstx_ctx_destroy(ctx)
+            (lib().fstx_ctx_release if self._shared else lib().fstx_ctx_destroy)(ctx)
 
     def __del__(self) -> None:
         try:

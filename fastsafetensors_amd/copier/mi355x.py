@@ -100,11 +100,12 @@ class MI355XFileCopier(CopierInterface):
         total = meta.size_bytes - first
         lead = self.data_at if self.layout == "direct" else 0
         gbuf = self.framework.alloc_tensor_memory(lead + total, self.device)
-        # The allocator may hand back memory that kernels already queued on the caller's
-        # stream still read (a buffer closed a moment ago).  The copy streams are not
-        # ordered after that stream, so let it drain before they write into the arena.
-        self.framework.synchronize(self.device)
         try:
+            # The allocator may hand back memory that kernels already queued on the caller's
+            # stream still read (a buffer closed a moment ago).  The copy streams are not
+            # ordered after that stream by themselves: make them wait for what it holds now
+            # (an event, not a device-wide synchronize: other streams of the caller keep running).
+            self.reader.order_after(self.framework.current_stream(self.device))
             done = 0
             while done < total:
                 length = min(total - done, max_copy_block_size)
@@ -155,7 +156,8 @@ class MI355XFileCopier(CopierInterface):
                 meta.data_length,
                 self._stream(),
             )
-            fw.synchronize(self.device)
+            # the window goes back to the allocator right away: its reuse is ordered after this
+            # kernel on the same stream, and by order_after() for the copy streams
             fw.shrink_tensor_memory(gbuf)
             arena, data_at = fresh, lead
 
@@ -181,7 +183,6 @@ class MI355XFileCopier(CopierInterface):
                 ],
                 self._stream(),
             )
-            fw.synchronize(self.device)
 
         tensors: Dict[str, TensorBase] = {}
         for name, frame in meta.tensors.items():
@@ -208,30 +209,61 @@ class MI355XFileCopier(CopierInterface):
                     raise Exception(
                         f"Online type conversion to larger sizes is not supported ({frame.dtype} -> {dtype})"
                     )
-                if frame.dtype.value not in _native.ELEM_TYPES or dtype.value not in _native.ELEM_TYPES:
-                    raise NotImplementedError(
-                        f"conversion on load from {frame.dtype} to {dtype} has no kernel "
-                        f"(supported: {sorted(_native.ELEM_TYPES)})"
-                    )
             if frame.dtype != dtype or (src_at + frame.data_offsets[0]) % PTR_ALIGN:
                 placed[name] = cursor
                 count = frame.nbytes * 8 // dtype_bits(frame.dtype)
                 cursor += _align_up(count * (want_bits if frame.dtype != dtype else dtype_bits(frame.dtype)) // 8, LINE_ALIGN)
         side = fw.alloc_side_memory(gbuf, cursor, self.device)
-        convert, copy = [], []
-        for name, at in placed.items():
+        # A source that is misaligned for its own element type (a header of odd length, or odd
+        # byte counts in front of it) is first moved to an aligned scratch slot: neither the
+        # conversion kernel nor the framework can read it in place.
+        staged: Dict[str, int] = {}
+        scratch_bytes = 0
+        for name in placed:
             frame = meta.tensors[name]
-            src = src_at + frame.data_offsets[0]
-            if frame.dtype != dtype:
-                count = frame.nbytes * 8 // dtype_bits(frame.dtype)
-                if count:
+            if frame.dtype != dtype and frame.nbytes and (src_at + frame.data_offsets[0]) % dtype_storage_align(frame.dtype):
+                staged[name] = scratch_bytes
+                scratch_bytes += _align_up(frame.nbytes, LINE_ALIGN)
+        scratch = fw.alloc_tensor_memory(scratch_bytes, self.device) if staged else None
+        try:
+            if staged:
+                _native.realign_copy_batch(
+                    [(scratch.get_base_address() + at, src_at + meta.tensors[n].data_offsets[0], meta.tensors[n].nbytes)
+                     for n, at in staged.items()],
+                    self._stream(),
+                )
+            convert, copy, by_framework = [], [], []
+            for name, at in placed.items():
+                frame = meta.tensors[name]
+                if not frame.nbytes:
+                    continue
+                src = scratch.get_base_address() + staged[name] if name in staged else src_at + frame.data_offsets[0]
+                if frame.dtype == dtype:
+                    copy.append((side.get_base_address() + at, src, frame.nbytes))
+                elif _native.convert_supported(frame.dtype.value, dtype.value):
+                    count = frame.nbytes * 8 // dtype_bits(frame.dtype)
                     convert.append((side.get_base_address() + at, src, count,
                                     _native.ELEM_TYPES[frame.dtype.value], _native.ELEM_TYPES[dtype.value]))
-            elif frame.nbytes:
-                copy.append((side.get_base_address() + at, src, frame.nbytes))
-        _native.convert_batch(convert, self._stream())
-        _native.realign_copy_batch(copy, self._stream())
-        fw.synchronize(self.device)
+                else:
+                    by_framework.append((name, at))
+            _native.convert_batch(convert, self._stream())
+            _native.realign_copy_batch(copy, self._stream())
+            # Pairs the conversion kernel does not cover (integer and bool tensors, fp8 sources)
+            # are converted on the GPU by the framework's own copy, as the reference converts
+            # every tensor (common.py:355-375).
+            for name, at in by_framework:
+                frame = meta.tensors[name]
+                count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                if name in staged:
+                    src_view = fw.view_tensor(scratch, staged[name], frame, self.device)
+                else:
+                    src_view = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)
+                out_frame = TensorFrame(dtype, frame.shape, [at, at + count * want_bits // 8],
+                                        frame.strides, frame.offsets, frame.sliced)
+                fw.copy_tensor(fw.view_tensor(side, at, out_frame, self.device), src_view)
+        finally:
+            if scratch is not None:
+                fw.free_tensor_memory(scratch, self.device)  # reuse is ordered after the kernels above on this stream
         tensors: Dict[str, TensorBase] = {}
         for name, frame in meta.tensors.items():
             if name in placed:
@@ -248,9 +280,7 @@ class MI355XFileCopier(CopierInterface):
         return tensors
 
     def _stream(self) -> int:
-        import torch
-
-        return torch.cuda.current_stream().cuda_stream
+        return self.framework.current_stream(self.device)
 
     def __del__(self) -> None:
         try:
@@ -267,6 +297,52 @@ def _default_numa_node(device: Device) -> int:
     return -1 if node is None or node < 0 else node
 
 
+def _open_reader(
+    device: Device,
+    max_threads: int = 16,
+    block_size_kb: Optional[int] = None,
+    n_streams: int = 0,
+    slots_per_thread: int = 0,
+    max_direct_reads: int = 0,
+    direct_read_kb: Optional[int] = None,
+    direct_ramp_kb: Optional[int] = None,
+    adaptive_depth: bool = False,
+    numa_node: Optional[int] = None,
+    shared_reader: bool = True,
+) -> _native.Reader:
+    block_kb = block_size_kb or int(os.environ.get("FSTX_BLOCK_KB", "4096"))
+    return _native.Reader(
+        device.index if device.index is not None else 0,
+        numa_node=_default_numa_node(device) if numa_node is None else numa_node,
+        n_threads=max_threads,
+        n_streams=n_streams,
+        block_bytes=block_kb * 1024,
+        slots_per_thread=slots_per_thread,
+        max_direct_reads=max_direct_reads,
+        direct_read_bytes=(direct_read_kb or int(os.environ.get("FSTX_DIRECT_READ_KB", "0"))) * 1024,
+        adaptive_depth=adaptive_depth,
+        direct_ramp_kb=direct_ramp_kb if direct_ramp_kb is not None else int(os.environ.get("FSTX_DIRECT_RAMP_KB", "0")),
+        shared=shared_reader,
+    )
+
+
+def hold_reader(device: str = "cuda:0", max_threads: int = 16, **kwargs) -> _native.Reader:
+    """Keep the process-wide read pipeline of this configuration alive until the returned
+    handle is closed.
+
+    Loaders created meanwhile with the same settings find its threads, streams and pinned
+    ring ready instead of building them again, and, above all, find the ring's pages already
+    mapped: the first touch of freshly pinned memory costs about 0.3 ms per MiB, which is
+    most of the overhead of loading a file of a few hundred MB.  For processes that load
+    many small files one after another (adapters, shards on demand).  ``kwargs`` are the
+    copier's own (``block_size_kb``, ``n_streams``, ...).
+    """
+    import torch
+
+    dev = torch.device(device)
+    return _open_reader(Device(DeviceType(dev.type), dev.index), max_threads=max_threads, shared_reader=True, **kwargs)
+
+
 @register_copier_constructor("mi355x")
 def new_mi355x_file_copier(
     device: Device,
@@ -280,12 +356,16 @@ def new_mi355x_file_copier(
     slots_per_thread: int = 0,
     max_direct_reads: int = 0,
     direct_read_kb: Optional[int] = None,
+    direct_ramp_kb: Optional[int] = None,
     adaptive_depth: bool = False,
     numa_node: Optional[int] = None,
+    shared_reader: bool = True,
     **kwargs,
 ) -> CopierConstructFunc:
     """One read pipeline (threads, pinned ring, streams) shared by every file of a
-    loader, as the reference shares one ``nogds_file_reader`` (``copier/nogds.py:107-116``).
+    loader, as the reference shares one ``nogds_file_reader`` (``copier/nogds.py:107-116``)
+    -- and, unless ``shared_reader=False``, by every loader of the process that is alive at
+    the same time and asks for the same settings; the last one to close frees it.
 
     ``bbuf_size_kb`` is accepted for signature compatibility; the ring is sized
     ``max_threads * slots_per_thread * block_size_kb`` instead, because 1 MiB
@@ -298,17 +378,10 @@ def new_mi355x_file_copier(
         raise Exception("[FAIL] no HIP device is visible to libfstx")
     read_mode = read_mode or os.environ.get("FSTX_READ_MODE", "auto")
     layout = layout or os.environ.get("FSTX_LAYOUT", "direct")
-    block_kb = block_size_kb or int(os.environ.get("FSTX_BLOCK_KB", "4096"))
-    reader = _native.Reader(
-        device.index if device.index is not None else 0,
-        numa_node=_default_numa_node(device) if numa_node is None else numa_node,
-        n_threads=max_threads,
-        n_streams=n_streams,
-        block_bytes=block_kb * 1024,
-        slots_per_thread=slots_per_thread,
-        max_direct_reads=max_direct_reads,
-        direct_read_bytes=(direct_read_kb or int(os.environ.get("FSTX_DIRECT_READ_KB", "0"))) * 1024,
-        adaptive_depth=adaptive_depth,
+    reader = _open_reader(
+        device, max_threads=max_threads, block_size_kb=block_size_kb, n_streams=n_streams,
+        slots_per_thread=slots_per_thread, max_direct_reads=max_direct_reads, direct_read_kb=direct_read_kb,
+        direct_ramp_kb=direct_ramp_kb, adaptive_depth=adaptive_depth, numa_node=numa_node, shared_reader=shared_reader,
     )
 
     def construct(metadata: SafeTensorsMetadata, device: Device, framework: FrameworkOpBase) -> CopierInterface:

@@ -89,6 +89,20 @@ int event_sync(event_t e) {
     return rc(hipEventSynchronize(static_cast<hipEvent_t>(e)), "hipEventSynchronize");
 }
 
+int stream_idle(stream_t s) {
+    hipError_t q = hipStreamQuery(static_cast<hipStream_t>(s));
+    if (q == hipSuccess) return 1;
+    if (q == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return rc(q, "hipStreamQuery");
+}
+
+int stream_wait_event(stream_t s, event_t e) {
+    return rc(hipStreamWaitEvent(static_cast<hipStream_t>(s), static_cast<hipEvent_t>(e), 0), "hipStreamWaitEvent");
+}
+
 int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stream_t s) {
     return rc(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice,
                              static_cast<hipStream_t>(s)),

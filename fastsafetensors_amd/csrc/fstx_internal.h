@@ -31,6 +31,8 @@ int event_destroy(event_t e);
 int event_record(event_t e, stream_t s);
 int event_ready(event_t e);                 // 1 done, 0 still running, <0 error
 int event_sync(event_t e);
+int stream_idle(stream_t s);                  // 1 nothing queued on s is still running, 0 busy, <0 error
+int stream_wait_event(stream_t s, event_t e); // work queued on s after this call waits for e's last record
 int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stream_t s);
 
 } // namespace fstx_dev

@@ -11,8 +11,10 @@
 //   * every request is cut into blocks of `block_bytes` on 4 KiB file
 //     boundaries; workers pull blocks from one FIFO, so a single large file
 //     is read by all workers at once;
-//   * each worker cycles through its own slots of a pinned ring that is
-//     allocated once per context; after the read it enqueues an asynchronous
+//   * each worker cycles through its own slots of a pinned ring (every worker
+//     allocates its slots itself, once, after binding to the node, so the ring
+//     is placed without touching the creating thread's memory policy and the
+//     sixteen allocations run side by side); after the read it enqueues an asynchronous
 //     host-to-device copy and an event on one of the shared copy streams and
 //     moves on to its next slot, so the copy of block k overlaps the read of
 //     block k+1 (the event is waited only when the slot comes round again);
@@ -234,7 +236,7 @@ class Gate {
 
 struct Counters {
     std::atomic<uint64_t> bytes_read{0}, bytes_copied{0}, blocks_buffered{0}, blocks_direct{0},
-        read_ns{0}, stage_ns{0}, slot_wait_ns{0}, direct_fallbacks{0};
+        read_ns{0}, stage_ns{0}, slot_wait_ns{0}, direct_fallbacks{0}, direct_reads{0};
 };
 
 } // namespace
@@ -242,7 +244,8 @@ struct Counters {
 struct fstx_ctx {
     fstx_config cfg{};
     uint64_t ring_bytes = 0;
-    char *ring = nullptr;
+    uint64_t slot_bytes = 0;
+    std::vector<char *> rings; // one pinned allocation per worker, made by the worker
     std::vector<fstx_dev::stream_t> streams;
     std::vector<std::vector<Slot>> slots; // [thread][slot]
     std::vector<std::thread> workers;
@@ -252,6 +255,9 @@ struct fstx_ctx {
     std::condition_variable q_cv;
     std::deque<Block> queue;
     std::deque<Staged> staged; // read by O_DIRECT, waiting for a worker to ship them (q_mutex)
+    uint64_t queue_bytes = 0;              // payload bytes of the blocks in `queue` (q_mutex)
+    uint32_t burst_runs = 0;               // O_DIRECT runs started since `queue` was last empty (q_mutex)
+    uint64_t ramp_bytes = 0;               // size of the first run of a burst
     uint64_t queue_pops = 0;               // blocks taken off `queue` so far (q_mutex)
     uint64_t head_verdict_for = ~0ull;     // value of queue_pops the cached verdict belongs to
     bool head_wants_direct = false;        // whether the block at the head of `queue` is to be read with O_DIRECT
@@ -259,6 +265,18 @@ struct fstx_ctx {
 
     std::mutex done_mutex;
     std::condition_variable done_cv;
+
+    // start-up handshake: every worker reports once its slots and events exist
+    std::mutex ready_mutex;
+    std::condition_variable ready_cv;
+    uint32_t ready = 0;
+    int ready_status = 0;
+
+    // fstx_ctx_order_after: one event, recorded on the caller's stream, awaited by the copy streams
+    std::mutex order_mutex;
+    fstx_dev::event_t order_event = nullptr;
+    uint64_t create_ns = 0;
+    bool no_copy = false, no_read = false; // FSTX_PROBE_*
 
     std::mutex table_mutex;
     std::map<int64_t, std::shared_ptr<FileEntry>> files;
@@ -322,6 +340,30 @@ bool block_is_cached(const FileEntry &f, uint64_t lo, uint64_t hi) {
     return (double)in >= kResidentEnough * (double)pages;
 }
 
+// Page-cache residency of one stretch of a file, asked once (mincore) and then queried per block.
+struct Residency {
+    std::vector<unsigned char> vec;
+    uint64_t lo = 0, hi = 0;
+    void probe(const FileEntry &f, uint64_t from, uint64_t to) {
+        if (!f.map) return;
+        lo = align_down(from, kPage);
+        hi = std::min(align_up(to, kPage), align_up(f.size, kPage));
+        if (hi <= lo) { hi = lo; return; }
+        vec.resize((size_t)((hi - lo) / kPage));
+        if (mincore(static_cast<char *>(f.map) + lo, hi - lo, vec.data()) != 0) vec.clear(), hi = lo;
+    }
+    // whether [a, b) lies in the probed stretch and is (nearly) all resident
+    bool cached(uint64_t a, uint64_t b) const {
+        a = align_down(a, kPage);
+        b = std::min(align_up(b, kPage), hi);
+        if (vec.empty() || a < lo || b <= a) return false;
+        size_t in = 0;
+        const size_t first = (size_t)((a - lo) / kPage), n = (size_t)((b - a) / kPage);
+        for (size_t i = 0; i < n; ++i) in += vec[first + i] & 1;
+        return (double)in >= kResidentEnough * (double)n;
+    }
+};
+
 struct Worker {
     fstx_ctx *ctx;
     uint32_t index;
@@ -366,13 +408,14 @@ struct Worker {
 
     // enqueue slot -> device for block b; payload sits at slot.host + at
     int64_t ship(const Block &b, Slot &slot, uint64_t at) {
+        ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
+        if (ctx->no_copy) return 0; // measuring the reads alone
         int64_t status = fstx_dev::copy_to_device_async(b.dev, slot.host + at, b.len, stream);
         if (status < 0) return status;
         slot.pending = true;
         status = fstx_dev::event_record(slot.ev, stream);
         b.req->stream_mask.fetch_or(1ull << stream_ix, std::memory_order_relaxed);
         ctx->ctr.bytes_copied.fetch_add(b.len, std::memory_order_relaxed);
-        ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
         return status;
     }
 
@@ -395,7 +438,8 @@ struct Worker {
         if (status < 0) return status;
         const uint64_t at = b.file_off % kPage;
         uint64_t t0 = now_ns();
-        int64_t got = pread_full(b.req->file->fd_buffered, slot->host + at, b.len, b.file_off);
+        int64_t got = ctx->no_read ? (int64_t)b.len
+                                   : pread_full(b.req->file->fd_buffered, slot->host + at, b.len, b.file_off);
         ctx->ctr.read_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
         if (got < 0) return got;
         if ((uint64_t)got < b.len) return -FSTX_E_SHORT_READ;
@@ -437,8 +481,10 @@ struct Worker {
             return true;
         }
         uint64_t t0 = now_ns();
-        int64_t got = pread_full(f.fd_direct, stage, want, window);
+        int64_t got = ctx->no_read ? (int64_t)std::min(want, align_up(f.size, kPage) - window)
+                                   : pread_full(f.fd_direct, stage, want, window);
         uint64_t t1 = now_ns();
+        ctx->ctr.direct_reads.fetch_add(1, std::memory_order_relaxed);
         release_token(got > 0 ? (uint64_t)got : 0);
         if (got == -EINVAL || got == -EFAULT || got == -EOPNOTSUPP) {
             f.direct_ok.store(false, std::memory_order_relaxed);
@@ -473,7 +519,10 @@ struct Worker {
         const Block &b = st.block;
         int64_t status = b.req->error.load(std::memory_order_relaxed);
         Slot *slot = nullptr;
-        if (status == 0 && (status = take_slot(&slot)) == 0) {
+        if (status == 0 && ctx->no_copy) { // measuring the reads alone: the bytes stay where the read left them
+            ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
+            ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
+        } else if (status == 0 && (status = take_slot(&slot)) == 0) {
             uint64_t t0 = now_ns();
             std::memcpy(slot->host, st.bytes, b.len);
             ctx->ctr.stage_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
@@ -505,6 +554,24 @@ struct Worker {
         return true;
     }
 
+    // called with q_mutex held: bytes the next O_DIRECT pread may cover.  The first read after
+    // the queue was empty is small, so that copies start early, and the following ones grow
+    // fourfold up to the full size; towards the end of what is queued the reads halve again,
+    // because the copy of the last read is the one stretch during which the storage idles.
+    uint64_t run_limit() const {
+        uint64_t limit = ctx->direct_bytes;
+        const uint64_t ramp = ctx->ramp_bytes;
+        if (ramp < limit) {
+            const uint32_t k = std::min(ctx->burst_runs, 16u);
+            const uint64_t up = ramp << (2 * k);
+            if ((up >> (2 * k)) == ramp && up < limit) limit = up;
+            const uint64_t down = std::max(ramp, ctx->queue_bytes / 2);
+            if (down < limit) limit = down;
+        }
+        const uint64_t bb = ctx->cfg.block_bytes;
+        return std::max(bb, align_down(limit, bb));
+    }
+
     void return_stage() {
         if (!stage) return;
         {
@@ -515,10 +582,35 @@ struct Worker {
         ctx->q_cv.notify_all();
     }
 
+    // The worker's share of the pinned ring and its events, made by the worker itself: it is
+    // bound to the node by then, so the memory is placed there without changing the policy of
+    // the thread that creates the context, and the workers allocate side by side.
+    int make_slots() {
+        void *p = nullptr;
+        int rc = fstx_dev::host_alloc(&p, ctx->slot_bytes * ctx->cfg.slots_per_thread);
+        if (rc < 0) return rc;
+        ctx->rings[index] = static_cast<char *>(p);
+        fstx_internal::note_bounce_bytes((int64_t)(ctx->slot_bytes * ctx->cfg.slots_per_thread));
+        for (uint32_t k = 0; k < ctx->cfg.slots_per_thread; ++k) {
+            Slot s;
+            s.host = ctx->rings[index] + k * ctx->slot_bytes;
+            if ((rc = fstx_dev::event_create(&s.ev)) < 0) return rc;
+            mine->push_back(s);
+        }
+        return 0;
+    }
+
     void run() {
         bind_thread_to_node(ctx->cfg.numa_node);
-        const int64_t dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
+        int64_t dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
         mine = &ctx->slots[index];
+        if (dev_rc == 0) dev_rc = make_slots();
+        {
+            std::lock_guard<std::mutex> lk(ctx->ready_mutex);
+            ++ctx->ready;
+            if (dev_rc < 0 && ctx->ready_status == 0) ctx->ready_status = (int)dev_rc;
+        }
+        ctx->ready_cv.notify_all();
         stream_ix = index % (uint32_t)ctx->streams.size();
         stream = ctx->streams[stream_ix];
         std::vector<Block> run;
@@ -573,24 +665,34 @@ struct Worker {
                 }
                 if (!have_staged) {
                     if (ctx->queue.empty()) break;
-                    run.push_back(std::move(ctx->queue.front()));
-                    ctx->queue.pop_front();
-                    ++ctx->queue_pops;
+                    const uint64_t limit = direct ? run_limit() : 0;
+                    auto pop = [&] {
+                        ctx->queue_bytes -= ctx->queue.front().len;
+                        run.push_back(std::move(ctx->queue.front()));
+                        ctx->queue.pop_front();
+                        ++ctx->queue_pops;
+                    };
+                    pop();
                     if (direct) {
-                        // extend the run with the blocks that follow it in the file
+                        // extend the run with the blocks that follow it in the file; in AUTO mode
+                        // only as far as the file is not in the page cache (one mincore call over
+                        // the stretch the run may cover)
+                        ++ctx->burst_runs;
+                        FileEntry &f = *run[0].req->file;
+                        Residency seen;
+                        if (f.mode == FSTX_READ_AUTO) seen.probe(f, run[0].file_off + run[0].len, run[0].file_off + limit);
                         uint64_t bytes = run[0].len + run[0].file_off % kPage;
                         while (!ctx->queue.empty()) {
                             const Block &nx = ctx->queue.front();
                             const Block &last = run.back();
-                            if (nx.req != last.req || nx.file_off != last.file_off + last.len ||
-                                bytes + nx.len > ctx->direct_bytes)
+                            if (nx.req != last.req || nx.file_off != last.file_off + last.len || bytes + nx.len > limit ||
+                                seen.cached(nx.file_off, nx.file_off + nx.len))
                                 break;
                             bytes += nx.len;
-                            run.push_back(std::move(ctx->queue.front()));
-                            ctx->queue.pop_front();
-                            ++ctx->queue_pops;
+                            pop();
                         }
                     }
+                    if (ctx->queue.empty()) ctx->burst_runs = 0; // the next read starts a new burst
                 }
             }
             if (have_staged) {
@@ -697,10 +799,10 @@ const char *fstx_strerror(int64_t code) {
 
 // ---- context -----------------------------------------------------------------
 
-int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
-    if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
-    *out = nullptr;
-    fstx_config cfg = *cfg_in;
+namespace {
+
+// defaults filled in, limits checked; 0 or a negative status
+int normalize(fstx_config &cfg) {
     if (cfg.n_threads == 0) cfg.n_threads = 8;
     if (cfg.n_streams == 0) cfg.n_streams = 4;
     if (cfg.block_bytes == 0) cfg.block_bytes = kDefaultBlock;
@@ -708,70 +810,96 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
     if (cfg.max_direct_reads == 0) cfg.max_direct_reads = adaptive_depth ? g_depth_hint.load() : 1;
     if (cfg.direct_read_bytes == 0) cfg.direct_read_bytes = 1ull << 30;
-    cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
-    if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 ||
-        cfg.slots_per_thread > 64)
+    if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 || cfg.slots_per_thread > 64 ||
+        (cfg.flags & ~(FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_NO_COPY | FSTX_PROBE_NO_READ)))
         return -FSTX_E_INVAL;
+    cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
+    if (cfg.direct_ramp_kb == 0) cfg.direct_ramp_kb = 64 * 1024;
     cfg.n_streams = std::min(cfg.n_streams, cfg.n_threads);
+    cfg.struct_size = sizeof(fstx_config);
+    return 0;
+}
+
+void free_parts(fstx_ctx *ctx) {
+    for (auto &per : ctx->slots)
+        for (Slot &s : per)
+            if (s.ev) fstx_dev::event_destroy(s.ev);
+    if (ctx->order_event) fstx_dev::event_destroy(ctx->order_event);
+    for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
+    for (char *r : ctx->rings)
+        if (r) {
+            fstx_dev::host_free(r);
+            fstx_internal::note_bounce_bytes(-(int64_t)(ctx->slot_bytes * ctx->cfg.slots_per_thread));
+        }
+}
+
+void stop_workers(fstx_ctx *ctx) {
+    {
+        std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        ctx->closing = true;
+    }
+    ctx->q_cv.notify_all();
+    for (std::thread &t : ctx->workers) t.join(); // workers drain the queue first
+}
+
+// contexts handed out by fstx_ctx_acquire
+struct Shared {
+    fstx_config cfg;
+    fstx_ctx *ctx;
+    uint64_t users;
+};
+std::mutex g_shared_mutex;
+std::vector<Shared> g_shared;
+
+bool same_config(const fstx_config &a, const fstx_config &b) {
+    return a.device_id == b.device_id && a.numa_node == b.numa_node && a.n_threads == b.n_threads &&
+           a.n_streams == b.n_streams && a.block_bytes == b.block_bytes && a.slots_per_thread == b.slots_per_thread &&
+           a.max_direct_reads == b.max_direct_reads && a.direct_read_bytes == b.direct_read_bytes && a.flags == b.flags &&
+           a.direct_ramp_kb == b.direct_ramp_kb;
+}
+
+} // namespace
+
+int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
+    if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
+    *out = nullptr;
+    const uint64_t t_start = now_ns();
+    fstx_config cfg = *cfg_in;
+    int rc = normalize(cfg);
+    if (rc < 0) return rc;
+    const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
 
     int n_dev = fstx_dev::device_count();
     if (n_dev < 0) return n_dev;
     if (cfg.device_id < 0 || cfg.device_id >= n_dev) return -FSTX_E_INVAL;
-    int rc = fstx_dev::set_device(cfg.device_id);
+    rc = fstx_dev::set_device(cfg.device_id);
     if (rc < 0) return rc;
 
     std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
     ctx->cfg = cfg;
     ctx->adaptive_depth = adaptive_depth;
+    ctx->no_copy = (cfg.flags & FSTX_PROBE_NO_COPY) != 0;
+    ctx->no_read = (cfg.flags & FSTX_PROBE_NO_READ) != 0;
     ctx->direct_bytes = cfg.direct_read_bytes;
+    ctx->ramp_bytes = std::max(cfg.block_bytes, align_down((uint64_t)cfg.direct_ramp_kb * 1024, cfg.block_bytes));
     // one staging buffer per read in flight plus one that is being emptied into the ring meanwhile
     ctx->stage_max = (adaptive_depth ? std::min(cfg.n_threads, 8u) : std::min(cfg.max_direct_reads, cfg.n_threads)) + 1;
     ctx->direct_gate.reset(new Gate(cfg.max_direct_reads, std::min(cfg.n_threads, 32u), adaptive_depth));
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
 
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
-    const uint64_t slot_bytes = cfg.block_bytes + kPage;
-    const uint64_t n_slots = (uint64_t)cfg.n_threads * cfg.slots_per_thread;
-    ctx->ring_bytes = slot_bytes * n_slots;
-    {
-        // allocate (and thereby place) the ring while this thread prefers the node
-        cpu_set_t saved;
-        bool restore = cfg.numa_node >= 0 && sched_getaffinity(0, sizeof saved, &saved) == 0;
-        if (cfg.numa_node >= 0) bind_thread_to_node(cfg.numa_node);
-        void *p = nullptr;
-        rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
-        if (restore) {
-            sched_setaffinity(0, sizeof saved, &saved);
-#ifdef SYS_set_mempolicy
-            (void)syscall(SYS_set_mempolicy, 0, nullptr, 0); // MPOL_DEFAULT
-#endif
-        }
-        if (rc < 0) return rc;
-        ctx->ring = static_cast<char *>(p);
-        fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
-    }
-    auto fail = [&](int code) {
-        for (auto &per : ctx->slots)
-            for (Slot &s : per)
-                if (s.ev) fstx_dev::event_destroy(s.ev);
-        for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
-        fstx_dev::host_free(ctx->ring);
-        fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
-        return code;
-    };
-    for (uint32_t i = 0; i < cfg.n_streams; ++i) {
-        fstx_dev::stream_t s = nullptr;
-        if ((rc = fstx_dev::stream_create(&s)) < 0) return fail(rc);
-        ctx->streams.push_back(s);
-    }
+    ctx->slot_bytes = cfg.block_bytes + kPage;
+    ctx->ring_bytes = ctx->slot_bytes * cfg.n_threads * cfg.slots_per_thread;
+    ctx->rings.assign(cfg.n_threads, nullptr);
     ctx->slots.resize(cfg.n_threads);
-    for (uint32_t t = 0; t < cfg.n_threads; ++t) {
-        for (uint32_t k = 0; k < cfg.slots_per_thread; ++k) {
-            Slot s;
-            s.host = ctx->ring + ((uint64_t)t * cfg.slots_per_thread + k) * slot_bytes;
-            if ((rc = fstx_dev::event_create(&s.ev)) < 0) return fail(rc);
-            ctx->slots[t].push_back(s);
-        }
+    for (uint32_t i = 0; i < cfg.n_streams && rc == 0; ++i) {
+        fstx_dev::stream_t s = nullptr;
+        if ((rc = fstx_dev::stream_create(&s)) == 0) ctx->streams.push_back(s);
+    }
+    if (rc == 0) rc = fstx_dev::event_create(&ctx->order_event);
+    if (rc < 0) {
+        free_parts(ctx.get());
+        return rc;
     }
     fstx_ctx *raw = ctx.release();
     for (uint32_t t = 0; t < cfg.n_threads; ++t) {
@@ -780,33 +908,85 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
             w.run();
         });
     }
-    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu", cfg.device_id,
+    {
+        // the workers allocate their shares of the ring; a context exists once all of them have
+        std::unique_lock<std::mutex> lk(raw->ready_mutex);
+        raw->ready_cv.wait(lk, [&] { return raw->ready == cfg.n_threads; });
+        rc = raw->ready_status;
+    }
+    if (rc < 0) {
+        stop_workers(raw);
+        free_parts(raw);
+        delete raw;
+        return rc;
+    }
+    raw->create_ns = now_ns() - t_start;
+    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu in %.2f ms", cfg.device_id,
                          cfg.n_threads, cfg.n_streams, (unsigned long long)cfg.block_bytes,
-                         (unsigned long long)raw->ring_bytes);
+                         (unsigned long long)raw->ring_bytes, raw->create_ns / 1e6);
     *out = raw;
     return 0;
 }
 
 int fstx_ctx_destroy(fstx_ctx *ctx) {
     if (!ctx) return -FSTX_E_INVAL;
-    {
-        std::lock_guard<std::mutex> lk(ctx->q_mutex);
-        ctx->closing = true;
-    }
-    ctx->q_cv.notify_all();
-    for (std::thread &t : ctx->workers) t.join(); // workers drain the queue first
+    stop_workers(ctx);
     if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->limit());
     fstx_dev::set_device(ctx->cfg.device_id);
     for (auto s : ctx->streams) fstx_dev::stream_sync(s);
-    for (auto &per : ctx->slots)
-        for (Slot &s : per) fstx_dev::event_destroy(s.ev);
-    for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
     for (auto &kv : ctx->files) release_file(*kv.second);
     for (char *p : ctx->stage_free) std::free(p);
-    fstx_dev::host_free(ctx->ring);
-    fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
+    free_parts(ctx);
     delete ctx;
     return 0;
+}
+
+int fstx_ctx_acquire(const fstx_config *cfg_in, fstx_ctx **out) {
+    if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
+    *out = nullptr;
+    fstx_config cfg = *cfg_in;
+    int rc = normalize(cfg);
+    if (rc < 0) return rc;
+    std::lock_guard<std::mutex> lk(g_shared_mutex);
+    for (Shared &s : g_shared)
+        if (same_config(s.cfg, cfg)) {
+            ++s.users;
+            *out = s.ctx;
+            return 0;
+        }
+    fstx_ctx *ctx = nullptr;
+    if ((rc = fstx_ctx_create(&cfg, &ctx)) < 0) return rc;
+    g_shared.push_back(Shared{cfg, ctx, 1});
+    *out = ctx;
+    return 0;
+}
+
+int fstx_ctx_release(fstx_ctx *ctx) {
+    if (!ctx) return -FSTX_E_INVAL;
+    {
+        std::lock_guard<std::mutex> lk(g_shared_mutex);
+        for (size_t i = 0; i < g_shared.size(); ++i)
+            if (g_shared[i].ctx == ctx) {
+                if (--g_shared[i].users > 0) return 0;
+                g_shared.erase(g_shared.begin() + (long)i);
+                break;
+            }
+    }
+    return fstx_ctx_destroy(ctx); // the last user, or a private context
+}
+
+int fstx_ctx_order_after(fstx_ctx *ctx, void *stream) {
+    if (!ctx) return -FSTX_E_INVAL;
+    std::lock_guard<std::mutex> lk(ctx->order_mutex);
+    int rc = fstx_dev::set_device(ctx->cfg.device_id);
+    if (rc < 0) return rc;
+    // Nothing running on the caller's stream: nothing to wait for.  (Worth asking: an event on
+    // an idle stream can still complete late, when that stream shares a hardware queue with a
+    // busy one.)
+    if (fstx_dev::stream_idle(stream) == 1) return 0;
+    rc = fstx_dev::event_record(ctx->order_event, stream);
+    for (size_t i = 0; i < ctx->streams.size() && rc == 0; ++i) rc = fstx_dev::stream_wait_event(ctx->streams[i], ctx->order_event);
+    return rc;
 }
 
 // ---- files ---------------------------------------------------------------------
@@ -841,6 +1021,7 @@ int64_t fstx_file_open(fstx_ctx *ctx, const char *path, int mode) {
 int fstx_file_close(fstx_ctx *ctx, int64_t file) {
     if (!ctx) return -FSTX_E_INVAL;
     std::shared_ptr<FileEntry> f;
+    bool idle = false;
     {
         std::lock_guard<std::mutex> lk(ctx->table_mutex);
         auto it = ctx->files.find(file);
@@ -848,8 +1029,20 @@ int fstx_file_close(fstx_ctx *ctx, int64_t file) {
         if (it->second->open_requests.load() != 0) return -EBUSY;
         f = it->second;
         ctx->files.erase(it);
+        idle = ctx->files.empty();
     }
     release_file(*f);
+    if (idle) {
+        // nothing is open any more: the staging buffers of the O_DIRECT reads (up to
+        // direct_read_bytes each) that are not on loan go back to the system until the next cold read
+        std::vector<char *> spare;
+        {
+            std::lock_guard<std::mutex> lq(ctx->q_mutex);
+            spare.swap(ctx->stage_free);
+            ctx->stage_made -= (uint32_t)spare.size();
+        }
+        for (char *p : spare) std::free(p);
+    }
     return 0;
 }
 
@@ -877,7 +1070,11 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
     // first byte, so that every block's O_DIRECT window fits one slot.
     std::vector<Block> blocks;
     if (length && req->error.load() == 0) {
-        const uint64_t bb = ctx->cfg.block_bytes;
+        // Small requests are cut into smaller blocks (at least 512 KiB, about 256 per request):
+        // a slot's pages are mapped at their first touch, which is slow for pinned memory, and a
+        // small load would otherwise spend longer touching the whole ring than copying.
+        uint64_t bb = ctx->cfg.block_bytes;
+        while (bb > (512u << 10) && bb % (2 * kPage) == 0 && bb * 256 > length) bb /= 2;
         const uint64_t origin = align_down(file_off, kPage);
         const uint64_t end = file_off + length;
         for (uint64_t lo = origin; lo < end; lo += bb) {
@@ -895,7 +1092,10 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
                 req->file->open_requests.fetch_sub(1);
                 return -FSTX_E_CLOSED;
             }
-            for (Block &b : blocks) ctx->queue.push_back(std::move(b));
+            for (Block &b : blocks) {
+                ctx->queue_bytes += b.len;
+                ctx->queue.push_back(std::move(b));
+            }
         }
         ctx->q_cv.notify_all();
     }
@@ -942,6 +1142,8 @@ int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
     out->slot_wait_ns = c.slot_wait_ns.load();
     out->direct_fallbacks = c.direct_fallbacks.load();
     out->direct_depth = ctx->direct_gate->limit();
+    out->direct_reads = c.direct_reads.load();
+    out->create_ns = ctx->create_ns;
     return 0;
 }
 

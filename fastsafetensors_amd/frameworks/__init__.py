@@ -146,6 +146,14 @@ class FrameworkOpBase(ABC):
     def synchronize(self, device: Device) -> None:
         return None
 
+    def current_stream(self, device: Device) -> int:
+        """Handle of the stream the calling thread's GPU work goes to (0: the null stream)."""
+        return 0
+
+    def synchronize_stream(self, device: Device) -> None:
+        """Wait for the work queued on the calling thread's stream only."""
+        return None
+
     def get_global_rank(self) -> int:
         return 0
 

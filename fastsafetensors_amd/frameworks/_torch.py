@@ -204,6 +204,9 @@ class TorchOp(FrameworkOpBase):
                 f"out of bound access: length={gbuf.get_length()}, request offset={byte_offset}, "
                 f"request length={nbytes}"
             )
+        if nbytes == 0:
+            # no bytes to alias, and a view at an offset that is odd for the dtype would be refused
+            return self.get_empty_tensor(frame.shape, frame.dtype, device)
         raw = gbuf.keepalive[byte_offset : byte_offset + nbytes]
         t = raw.view(dtype_convert[frame.dtype]).view(self.get_native_shape(frame.dtype, frame.shape))
         return TorchTensor(device, frame.dtype, t)
@@ -391,6 +394,13 @@ class TorchOp(FrameworkOpBase):
     def synchronize(self, device: Device) -> None:
         if device.type != DeviceType.CPU and torch.cuda.is_available():
             torch.cuda.synchronize()
+
+    def current_stream(self, device: Device) -> int:
+        return torch.cuda.current_stream(device.as_str()).cuda_stream
+
+    def synchronize_stream(self, device: Device) -> None:
+        if device.type != DeviceType.CPU and torch.cuda.is_available():
+            torch.cuda.current_stream(device.as_str()).synchronize()
 
     def get_device_name(self, index: int) -> str:
         try:

@@ -125,6 +125,10 @@ class BaseSafeTensorsFileLoader:
                     mine.append(factory)
             for factory in mine:
                 factory.wait_io(dtype=dtype, noalign=False)
+            # wait_io may have queued realign / convert kernels on this thread's stream: the
+            # tensors are complete when this call returns, as after the reference's synchronous copies
+            self.framework.synchronize_stream(self.device)
+            return FilesBufferOnDevice(factories, pg=self.pg, framework=self.framework)
         except Exception:
             # leave no arena and no in-flight read behind
             for factory in mine:
@@ -134,7 +138,6 @@ class BaseSafeTensorsFileLoader:
                 finally:
                     factory.free_dev_ptrs()
             raise
-        return FilesBufferOnDevice(factories, pg=self.pg, framework=self.framework)
 
 
 class SafeTensorsFileLoader(BaseSafeTensorsFileLoader):

@@ -157,7 +157,10 @@ class PipelineParallel:
                 try:
                     yield from self._tensors_of(item)
                     if item.fb.framework is not None:
-                        item.fb.framework.synchronize(self.loader.device)  # copies done before the source goes
+                        # the copies out of the batch ran on this thread's stream: they must be done
+                        # before the batch's memory goes back to the allocator (the producer thread
+                        # allocates from it); other streams of the caller are left alone
+                        item.fb.framework.synchronize_stream(self.loader.device)
                 finally:
                     item.fb.close()
                     pending = None

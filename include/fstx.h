@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define FSTX_ABI_VERSION 1
+#define FSTX_ABI_VERSION 2
 
 /* status codes beyond errno */
 #define FSTX_E_BASE 10000
@@ -67,12 +67,27 @@ typedef struct fstx_config {
     uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 1)      */
     uint64_t direct_read_bytes; /* bytes one O_DIRECT pread covers: a run of consecutive blocks,
                                    multiple of block_bytes (0 = 1 GiB)                           */
-    uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH                                              */
-    uint32_t reserved;
+    uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_*                               */
+    uint32_t direct_ramp_kb; /* KiB of the first O_DIRECT pread after the queue was empty; the next
+                                ones are 4x, 16x .. as large up to direct_read_bytes, and towards the
+                                end of the queued bytes they halve down to this size again, so that
+                                the copy of one read overlaps the next read from the start and only a
+                                small last read is copied with the storage idle (0 = 64 MiB; a value
+                                >= direct_read_bytes / 1024 keeps every read at full size)        */
 } fstx_config;
 
 /* fstx_config.flags: steer max_direct_reads while reading (start value = max_direct_reads) */
 #define FSTX_ADAPTIVE_DEPTH 1u
+/* Measurement contexts: the same threads, queue, request sizes and ring, with one stage left
+ * out, so that the rate of the other stage alone can be put next to a load's.  The bytes
+ * that arrive in device memory are unspecified with either flag.
+ *   NO_COPY  reads run (O_DIRECT runs into staging, page-cache reads into the ring), nothing
+ *            is moved to the ring by memcpy or to the device: what the storage delivers to
+ *            this engine's request pattern;
+ *   NO_READ  no pread: every block's ring slot is sent to the device as it is: what the
+ *            ring -> HBM copies deliver with this engine's slots, streams and threads. */
+#define FSTX_PROBE_NO_COPY 2u
+#define FSTX_PROBE_NO_READ 4u
 
 typedef struct fstx_metrics {
     uint64_t bounce_buffer_bytes; /* pinned ring bytes currently allocated by this context       */
@@ -85,6 +100,8 @@ typedef struct fstx_metrics {
     uint64_t slot_wait_ns;        /* summed over workers: waiting for a ring slot's last copy    */
     uint64_t direct_fallbacks;    /* blocks that asked for O_DIRECT but were read buffered       */
     uint64_t direct_depth;        /* O_DIRECT preads currently allowed in flight                 */
+    uint64_t direct_reads;        /* O_DIRECT preads issued (each covers a run of blocks)        */
+    uint64_t create_ns;           /* what fstx_ctx_create took: threads, ring, streams, events   */
 } fstx_metrics;
 
 /* ---- library-wide helpers ------------------------------------------------ */
@@ -130,6 +147,26 @@ int fstx_ctx_create(const fstx_config *cfg, fstx_ctx **out);
 /* Drain outstanding work, join the workers, free ring, streams and events.
  * ~nogds_file_reader (cpp/ext.cpp:778-806). */
 int fstx_ctx_destroy(fstx_ctx *ctx);
+
+/* A context shared by everyone in the process who asks for the same configuration: the
+ * first call creates it, later calls with an equal fstx_config (after defaults) get the same
+ * context and raise its use count; fstx_ctx_release drops the count and destroys the context
+ * with the last user, so the pinned ring is gone when nobody holds a reader
+ * (fstx_bounce_buffer_bytes() == 0 again).  Loaders that are alive at the same time thereby
+ * share one set of threads, one ring and one set of streams, as the files of one loader share
+ * one nogds_file_reader in the reference (copier/nogds.py:107-116).  Requests of different
+ * users go through one FIFO.  A context from fstx_ctx_create is private; releasing it
+ * destroys it. */
+int fstx_ctx_acquire(const fstx_config *cfg, fstx_ctx **out);
+int fstx_ctx_release(fstx_ctx *ctx);
+
+/* Order the context's copy streams after the work that is queued on `stream` right now:
+ * copies of requests submitted after this call start only when that work has finished.  A
+ * caller whose allocator hands out device memory that kernels on `stream` may still be
+ * using calls this before fstx_submit_read instead of synchronizing the device.  (The
+ * reference has no counterpart: its copies are synchronous cudaMemcpy calls on the null
+ * stream, cpp/ext.cpp:693-705.) */
+int fstx_ctx_order_after(fstx_ctx *ctx, void *stream);
 
 /* Open a file for reading in `mode`; returns a file handle >= 1.
  * The reference's Python opens the fd itself (copier/nogds.py:26-31); here the

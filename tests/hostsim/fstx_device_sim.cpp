@@ -90,6 +90,16 @@ extern "C" {
 void fstx_sim_set_copy_delay_us(int us) { g_copy_delay_us.store(us); }
 void fstx_sim_fail_copy_after(int64_t n) { g_fail_copy_after.store(n); }
 int64_t fstx_sim_pinned_live(void) { return g_pinned_live.load(); }
+// a caller-side stream: created here, handed to fstx_ctx_order_after as its `stream`
+void *fstx_sim_stream_create(void) { return new SimStream; }
+void fstx_sim_stream_destroy(void *s) { delete static_cast<SimStream *>(s); }
+// queue a task that sleeps and then writes `value` to *flag
+void fstx_sim_stream_sleep_then_set(void *s, int us, volatile int *flag, int value) {
+    static_cast<SimStream *>(s)->push([=] {
+        std::this_thread::sleep_for(std::chrono::microseconds(us));
+        *flag = value;
+    });
+}
 }
 
 namespace fstx_dev {
@@ -156,6 +166,25 @@ int event_sync(event_t e) {
     std::unique_lock<std::mutex> lk(ev->m);
     uint64_t target = ev->recorded;
     ev->cv.wait(lk, [&] { return ev->completed >= target; });
+    return 0;
+}
+int stream_idle(stream_t s) {
+    SimStream *st = static_cast<SimStream *>(s);
+    std::lock_guard<std::mutex> lk(st->m);
+    return st->finished >= st->submitted ? 1 : 0;
+}
+int stream_wait_event(stream_t s, event_t e) {
+    // the waiting stream stalls until the record that is the event's latest right now has run
+    SimEvent *ev = static_cast<SimEvent *>(e);
+    uint64_t gen;
+    {
+        std::lock_guard<std::mutex> lk(ev->m);
+        gen = ev->recorded;
+    }
+    static_cast<SimStream *>(s)->push([ev, gen] {
+        std::unique_lock<std::mutex> lk(ev->m);
+        ev->cv.wait(lk, [&] { return ev->completed >= gen; });
+    });
     return 0;
 }
 int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stream_t s) {

@@ -21,6 +21,9 @@
 #include "fstx.h"
 
 extern "C" void fstx_sim_set_copy_delay_us(int us);
+extern "C" void *fstx_sim_stream_create(void);
+extern "C" void fstx_sim_stream_destroy(void *s);
+extern "C" void fstx_sim_stream_sleep_then_set(void *s, int us, volatile int *flag, int value);
 
 int main(int argc, char **argv) {
     if (argc < 2) return 2;
@@ -53,8 +56,16 @@ int main(int argc, char **argv) {
         cfg.slots_per_thread = 1 + round % 2;
         cfg.direct_read_bytes = round == 1 ? 0 : cfg.block_bytes * 3;
         cfg.flags = round == 2 ? FSTX_ADAPTIVE_DEPTH : 0;
-        fstx_ctx *ctx = nullptr;
-        if (fstx_ctx_create(&cfg, &ctx) != 0) return 3;
+        cfg.direct_ramp_kb = round == 0 ? 4 : 0;
+        fstx_ctx *ctx = nullptr, *again = nullptr;
+        // odd rounds go through the shared table: two users of one context
+        if (round % 2) {
+            if (fstx_ctx_acquire(&cfg, &ctx) != 0 || fstx_ctx_acquire(&cfg, &again) != 0 || again != ctx) return 3;
+        } else if (fstx_ctx_create(&cfg, &ctx) != 0) {
+            return 3;
+        }
+        void *foreign = fstx_sim_stream_create();
+        volatile int flag = 0;
         std::vector<std::thread> callers;
         for (int c = 0; c < 3; ++c) {
             callers.emplace_back([&, c] {
@@ -68,6 +79,10 @@ int main(int argc, char **argv) {
                 while (at < size) {
                     uint64_t len = 1 + rng() % (size / 5 + 1);
                     if (at + len > size) len = size - at;
+                    if (rng() % 4 == 0) {
+                        fstx_sim_stream_sleep_then_set(foreign, 50, &flag, c);
+                        if (fstx_ctx_order_after(ctx, foreign) != 0) bad++;
+                    }
                     int64_t r = fstx_submit_read(ctx, file, at, len, dev.data(), dev.size(), at + 7);
                     if (r < 0) { bad++; break; }
                     reqs.push_back(r);
@@ -84,7 +99,9 @@ int main(int argc, char **argv) {
         fstx_metrics m;
         fstx_get_metrics(ctx, &m);
         if (m.bytes_copied != 3 * size) bad++;
-        if (fstx_ctx_destroy(ctx) != 0) bad++;
+        fstx_sim_stream_destroy(foreign); // drains it: the stand-in's events must outlive their records
+        if (again && fstx_ctx_release(again) != 0) bad++;
+        if ((again ? fstx_ctx_release(ctx) : fstx_ctx_destroy(ctx)) != 0) bad++;
     }
     if (fstx_bounce_buffer_bytes() != 0) bad++;
     std::printf("hostsim_driver: %s\n", bad.load() ? "MISMATCH" : "ok");

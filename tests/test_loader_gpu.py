@@ -271,7 +271,7 @@ def test_duplicate_key_across_files(golden, tmp_path):
     with pytest.raises(Exception, match="must be unique"):
         loader.copy_files_to_device()
     loader.close()
-    get_framework_op("pytorch").mem_used = 0  # the failed FilesBufferOnDevice never owned the buffers
+    assert_clean()  # the arenas of both files went back although no FilesBufferOnDevice ever owned them
 
 
 def test_full_size_c1_and_c2(data_dir):

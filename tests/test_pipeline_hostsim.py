@@ -35,6 +35,9 @@ def sim():
     lib.fstx_sim_set_copy_delay_us.argtypes = [ctypes.c_int]
     lib.fstx_sim_fail_copy_after.argtypes = [ctypes.c_int64]
     lib.fstx_sim_pinned_live.restype = ctypes.c_int64
+    lib.fstx_sim_stream_create.restype = ctypes.c_void_p
+    lib.fstx_sim_stream_destroy.argtypes = [ctypes.c_void_p]
+    lib.fstx_sim_stream_sleep_then_set.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
     lib.fstx_sim_set_copy_delay_us(30)
     return lib
 
@@ -48,13 +51,17 @@ def blob(tmp_path_factory):
 
 
 def make_ctx(sim, **kw):
-    cfg = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, kw.get("threads", 4), kw.get("streams", 2),
-                             kw.get("block", 64 * 1024), kw.get("slots", 2), kw.get("depth", 0),
-                             kw.get("direct_bytes", 0), kw.get("flags", 0), 0)
+    cfg = make_cfg(**kw)
     ctx = ctypes.c_void_p()
-    rc = sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(ctx))
+    rc = (sim.fstx_ctx_acquire if kw.get("shared") else sim.fstx_ctx_create)(ctypes.byref(cfg), ctypes.byref(ctx))
     assert rc == 0, rc
     return ctx
+
+
+def make_cfg(**kw):
+    return _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, kw.get("threads", 4), kw.get("streams", 2),
+                              kw.get("block", 64 * 1024), kw.get("slots", 2), kw.get("depth", 0),
+                              kw.get("direct_bytes", 0), kw.get("flags", 0), kw.get("ramp_kb", 0))
 
 
 def metrics(sim, ctx):
@@ -235,6 +242,139 @@ def test_destroy_with_requests_in_flight(sim, blob):
     sim.fstx_sim_set_copy_delay_us(30)
     assert np.array_equal(dev[:400_000], data[:400_000])
     assert sim.fstx_bounce_buffer_bytes() == 0
+
+
+def test_shared_contexts_are_counted(sim, blob):
+    """fstx_ctx_acquire: equal configurations share one context, the last release frees it."""
+    path, data = blob
+    a = make_ctx(sim, shared=True, threads=3)
+    b = make_ctx(sim, shared=True, threads=3)
+    c = make_ctx(sim, shared=True, threads=2)
+    private = make_ctx(sim, threads=3)
+    assert a.value == b.value and c.value != a.value and private.value != a.value
+    ring = lambda t: t * 2 * (64 * 1024 + 4096)
+    assert sim.fstx_bounce_buffer_bytes() == ring(3) + ring(2) + ring(3)
+    # two users at once, from two threads
+    import threading
+    devs = [np.zeros(data.size, dtype=np.uint8) for _ in range(2)]
+    def user(ctx, dev):
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, req) == data.size
+        assert sim.fstx_file_close(ctx, f) == 0
+    ts = [threading.Thread(target=user, args=(ctx, dev)) for ctx, dev in zip((a, b), devs)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert all(np.array_equal(d, data) for d in devs)
+    assert sim.fstx_ctx_release(a) == 0
+    assert sim.fstx_bounce_buffer_bytes() == ring(3) + ring(2) + ring(3)  # b still holds it
+    dev = np.zeros(1000, dtype=np.uint8)
+    f = sim.fstx_file_open(b, path.encode(), _native.READ_BUFFERED)
+    assert sim.fstx_wait_read(b, sim.fstx_submit_read(b, f, 5, 1000, dev.ctypes.data, 1000, 0)) == 1000
+    assert np.array_equal(dev, data[5:1005])
+    assert sim.fstx_ctx_release(b) == 0 and sim.fstx_ctx_release(c) == 0
+    assert sim.fstx_ctx_release(private) == 0  # a private context: release destroys it
+    assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+    # after the last release the next acquire builds a new context
+    d = make_ctx(sim, shared=True, threads=3)
+    assert sim.fstx_ctx_release(d) == 0 and sim.fstx_bounce_buffer_bytes() == 0
+
+
+def test_order_after_holds_the_copies_back(sim, blob):
+    """fstx_ctx_order_after: copies of later requests start only when the work that was
+    queued on the caller's stream at the call has run."""
+    path, data = blob
+    ctx = make_ctx(sim, threads=3, streams=3)
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+    theirs = sim.fstx_sim_stream_create()
+    flag = ctypes.c_int(0)
+    dev = np.zeros(200_000, dtype=np.uint8)
+    sim.fstx_sim_stream_sleep_then_set(theirs, 150_000, ctypes.byref(flag), 7)
+    assert sim.fstx_ctx_order_after(ctx, theirs) == 0
+    req = sim.fstx_submit_read(ctx, f, 0, dev.size, dev.ctypes.data, dev.size, 0)
+    import time
+    time.sleep(0.05)
+    assert flag.value == 0 and not dev.any()  # the reads are done by now, the copies still wait
+    assert sim.fstx_wait_read(ctx, req) == dev.size
+    assert flag.value == 7 and np.array_equal(dev, data[: dev.size])
+    # work queued on their stream after the call does not hold anything back
+    sim.fstx_sim_stream_sleep_then_set(theirs, 400_000, ctypes.byref(flag), 9)
+    req = sim.fstx_submit_read(ctx, f, 10, 1000, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == 1000 and flag.value == 7
+    assert sim.fstx_ctx_order_after(None, theirs) == -_native_code("INVAL")
+    sim.fstx_sim_stream_destroy(theirs)  # joins the stream's thread: flag is 9 afterwards
+    assert flag.value == 9
+    sim.fstx_ctx_destroy(ctx)
+
+
+def test_direct_reads_ramp_up_and_down(sim, blob):
+    """O_DIRECT runs: small first, growing fourfold to the full size, halving towards the end of
+    what is queued; a ramp size at or above the full size keeps every read at full size."""
+    path, data = blob
+    dev = np.zeros(data.size, dtype=np.uint8)
+    counts = {}
+    for label, ramp_kb in (("ramped", 64), ("fixed", 4096)):
+        ctx = make_ctx(sim, block=64 * 1024, threads=4, direct_bytes=4 << 20, ramp_kb=ramp_kb)
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_DIRECT)
+        dev[:] = 0
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, req) == data.size and np.array_equal(dev, data)
+        m = metrics(sim, ctx)
+        counts[label] = (m.direct_reads, m.direct_fallbacks)
+        sim.fstx_file_close(ctx, f)
+        sim.fstx_ctx_destroy(ctx)
+    if counts["fixed"][1] == 0:  # the filesystem took O_DIRECT
+        # 9,000,011 bytes in runs of 4 MiB: 3 reads; ramped: 64K, 256K, 1M, then halves of the rest down to 64K
+        assert counts["fixed"][0] == 3
+        assert 8 <= counts["ramped"][0] <= 14, counts
+
+
+def test_probe_contexts_leave_out_one_stage(sim, blob):
+    path, data = blob
+    for mode in (_native.READ_BUFFERED, _native.READ_DIRECT):
+        # NO_COPY: the reads run, device memory is not written
+        ctx = make_ctx(sim, flags=_native.PROBE_NO_COPY, direct_bytes=1 << 20)
+        f = sim.fstx_file_open(ctx, path.encode(), mode)
+        dev = np.full(data.size, 0xEE, dtype=np.uint8)
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, req) == data.size
+        m = metrics(sim, ctx)
+        assert m.bytes_read == data.size and m.bytes_copied == 0 and (dev == 0xEE).all()
+        sim.fstx_ctx_destroy(ctx)
+        # NO_READ: every block is copied, no byte comes from the file
+        ctx = make_ctx(sim, flags=_native.PROBE_NO_READ, direct_bytes=1 << 20)
+        f = sim.fstx_file_open(ctx, path.encode(), mode)
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, req) == data.size
+        m = metrics(sim, ctx)
+        assert m.bytes_copied == data.size and m.read_ns < 50_000_000
+        sim.fstx_ctx_destroy(ctx)
+    bad = make_cfg(flags=64)
+    out = ctypes.c_void_p()
+    assert sim.fstx_ctx_create(ctypes.byref(bad), ctypes.byref(out)) == -_native_code("INVAL")
+
+
+def test_auto_mode_reads_cached_stretches_from_the_cache(sim, tmp_path):
+    """AUTO: an O_DIRECT run stops at the first block that sits in the page cache."""
+    path = str(tmp_path / "partly.bin")
+    data = np.random.default_rng(5).integers(0, 256, 6 << 20, dtype=np.uint8)
+    data.tofile(path)
+    fd = os.open(path, os.O_RDONLY)
+    os.fsync(fd)
+    os.posix_fadvise(fd, 0, 0, os.POSIX_FADV_DONTNEED)
+    os.pread(fd, 2 << 20, 2 << 20)  # the middle third becomes resident
+    os.close(fd)
+    ctx = make_ctx(sim, block=256 * 1024, threads=3, direct_bytes=16 << 20, ramp_kb=16 << 10)
+    f = sim.fstx_file_open(ctx, path.encode(), _native.READ_AUTO)
+    dev = np.zeros(data.size, dtype=np.uint8)
+    req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+    assert sim.fstx_wait_read(ctx, req) == data.size and np.array_equal(dev, data)
+    m = metrics(sim, ctx)
+    if m.blocks_direct:  # the filesystem took O_DIRECT and the drop emptied the cache
+        # (read-ahead may have pulled in a little more than the 2 MiB that were read)
+        assert 8 <= m.blocks_buffered <= 14 and m.blocks_direct + m.blocks_buffered == 24, (m.blocks_direct, m.blocks_buffered)
+        assert m.direct_reads == 2
+    sim.fstx_ctx_destroy(ctx)
 
 
 @pytest.mark.parametrize("binary", ["hostsim_tsan.bin", "hostsim_asan.bin"])

@@ -1,0 +1,250 @@
+# SPDX-License-Identifier: Apache-2.0
+"""GPU tests of how the loader sits next to a caller's other GPU work and other loaders:
+stream ordering instead of device-wide synchronization, the process-wide shared reader,
+adaptive O_DIRECT depth, and the corners of the header rules that only show on a device
+(empty tensors at odd offsets, conversions the kernel has no pair for)."""
+import json
+import os
+import struct
+import time
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import load_file
+
+from fastsafetensors_amd import DType, SafeTensorsFileLoader, SingleGroup, _native, checkpoints as ck, hold_reader
+from fastsafetensors_amd.frameworks import get_framework_op
+from oracle import st_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev_bytes(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().reshape(-1).view(torch.uint8).cpu().numpy()
+
+
+def assert_clean():
+    assert get_framework_op("pytorch").get_mem_used() == 0
+    assert _native.get_cpp_metrics().bounce_buffer_bytes == 0
+
+
+def busy_kernel(ms: float) -> None:
+    """Queue a kernel that spins for about ``ms`` milliseconds on the current stream and then
+    ends by itself (torch's own test helper; calibrated once)."""
+    global _CYCLES_PER_MS
+    if _CYCLES_PER_MS is None:
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda._sleep(1_000_000)
+        torch.cuda.synchronize()
+        a.record()
+        torch.cuda._sleep(20_000_000)
+        b.record()
+        torch.cuda.synchronize()
+        _CYCLES_PER_MS = 20_000_000 / a.elapsed_time(b)
+    torch.cuda._sleep(int(ms * _CYCLES_PER_MS))
+
+
+_CYCLES_PER_MS = None
+
+
+def write_raw(path, entries, pad_to=8):
+    """A safetensors file written by hand: ``entries`` = [(name, dtype tag, shape, bytes)] in file order."""
+    table, at = {}, 0
+    for name, tag, shape, raw in entries:
+        table[name] = {"dtype": tag, "shape": list(shape), "data_offsets": [at, at + len(raw)]}
+        at += len(raw)
+    js = json.dumps(table, separators=(",", ":")).encode()
+    js += b" " * (-(8 + len(js)) % pad_to)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(js)) + js + b"".join(e[3] for e in entries))
+
+
+def test_load_does_not_wait_for_other_streams(golden, monkeypatch):
+    """A long kernel on a side stream of the caller: the load does not wait for it.  Two
+    checks.  (1) No device-wide synchronize is called anywhere on the path, in either layout.
+    (2) A load that launches no kernel (direct layout, aligned file) is back while the side
+    kernel still runs.  (A load that does launch kernels is ordered by the runtime, not by the
+    loader: null-stream work waits for every stream, and two streams may share one of the
+    few hardware queues.)"""
+    path = golden("tiny_gpt2.safetensors")
+    h = orc.parse_file(path)
+    side, mine = torch.cuda.Stream(), torch.cuda.Stream()
+    done = torch.cuda.Event()
+    busy_kernel(1.0)  # calibrate
+    torch.cuda.synchronize()
+
+    def refuse():
+        raise AssertionError("torch.cuda.synchronize() called on the load path")
+
+    with torch.cuda.stream(side):
+        busy_kernel(1500)  # about 1.5 s, finishes by itself
+        done.record()
+    t0 = time.perf_counter()
+    got = {}
+    with torch.cuda.stream(mine), monkeypatch.context() as mp:
+        mp.setattr(torch.cuda, "synchronize", refuse)
+        for layout in ("direct", "window"):
+            loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4, layout=layout)
+            loader.add_filenames({0: [path]})
+            bufs = loader.copy_files_to_device()
+            if layout == "direct":
+                assert not done.query(), f"the load came back only after the side stream's kernel ({time.perf_counter() - t0:.2f} s)"
+            got[layout] = {name: bufs.get_tensor(name).clone() for name in h.tensors}
+            mine.synchronize()
+            bufs.close()
+            loader.close()
+    side.synchronize()
+    for layout, tensors in got.items():
+        for name, t in tensors.items():
+            assert np.array_equal(dev_bytes(t), orc.tensor_bytes(path, h, name)), (layout, name)
+    got.clear()
+    assert_clean()
+
+
+def test_arena_reuse_is_ordered_after_the_callers_stream(golden, tmp_path):
+    """The allocator hands a closed buffer's memory to the next file; the copy streams must not
+    write it while a kernel queued earlier on the caller's stream still reads it."""
+    path = str(tmp_path / "big.safetensors")
+    n = 48 << 20
+    payload = torch.arange(n // 8, dtype=torch.int64)
+    write_raw(path, [("x", "I64", [n // 8], payload.numpy().tobytes())])
+    want_sum = int(payload.sum())
+    loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=8)
+    for _ in range(4):
+        loader.add_filenames({0: [path]})
+        bufs = loader.copy_files_to_device()
+        x = bufs.get_tensor("x")
+        busy_kernel(30)                            # the reduction below starts 30 ms from now ...
+        total = x.sum()                            # ... and reads the arena
+        bufs.close()                               # arena back to the allocator while that work is queued
+        loader.reset()
+        loader.add_filenames({0: [golden("tiny_gpt2.safetensors"), path]})
+        again = loader.copy_files_to_device()       # very likely reuses the block
+        assert int(total.item()) == want_sum
+        assert int(again.get_tensor("x").sum().item()) == want_sum
+        again.close()
+        loader.reset()
+    loader.close()
+    assert_clean()
+
+
+def test_shared_reader_lives_as_long_as_someone_holds_it(golden):
+    path = golden("a.safetensors")
+    ring = 4 * 2 * (4096 * 1024 + 4096)
+    a = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)
+    assert _native.bounce_buffer_bytes() == ring
+    b = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)          # same settings: same reader
+    c = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4, shared_reader=False)
+    assert _native.bounce_buffer_bytes() == 2 * ring
+    for ld in (a, b, c):
+        ld.add_filenames({0: [path]})
+        bufs = ld.copy_files_to_device()
+        assert torch.equal(bufs.get_tensor("a0").cpu()[:, 0], torch.arange(16, dtype=torch.float16))
+        bufs.close()
+    a.close()
+    c.close()
+    assert _native.bounce_buffer_bytes() == ring
+    b.close()
+    assert_clean()
+    # a held reader keeps threads and ring for loaders that come and go
+    hold = hold_reader(DEV, max_threads=4)
+    created = hold.metrics().create_ns
+    for _ in range(3):
+        ld = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)
+        assert ld.copier_constructor.reader.metrics().create_ns == created  # the same context
+        ld.add_filenames({0: [path]})
+        ld.copy_files_to_device().close()
+        ld.close()
+        assert _native.bounce_buffer_bytes() == ring
+    hold.close()
+    assert_clean()
+
+
+def test_adaptive_depth_and_small_direct_reads(tmp_path):
+    """O_DIRECT with many small reads in flight and the depth steered while reading -- the
+    setting for storage that wants a deep queue -- byte-exact against the oracle."""
+    cfg = ck.configs(0.08)["C3"]
+    files = [r["path"] for r in ck.write_config(cfg, str(tmp_path / "c3"))]
+    total = sum(os.path.getsize(f) for f in files)
+    loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=8, read_mode="direct", adaptive_depth=True,
+                                   direct_read_kb=1024, block_size_kb=512, shared_reader=False)
+    loader.add_filenames({0: files})
+    bufs = loader.copy_files_to_device()
+    m = loader.copier_constructor.reader.metrics()
+    for path in files:
+        h = orc.parse_file(path)
+        for name in h.tensors:
+            assert np.array_equal(dev_bytes(bufs.get_tensor(name)), orc.tensor_bytes(path, h, name)), name
+    assert m.direct_depth >= 1
+    if m.direct_fallbacks == 0:  # the filesystem took O_DIRECT
+        assert m.blocks_direct > 0 and m.blocks_buffered == 0
+        assert total // (1 << 20) <= m.direct_reads <= m.blocks_direct  # reads of at most 1 MiB
+    bufs.close()
+    loader.close()
+    assert_clean()
+
+
+def test_empty_wide_tensor_at_an_odd_offset(tmp_path):
+    """An empty F32 / I64 tensor that sits after an odd number of bytes: there is nothing to
+    view, and a view at that offset would not be legal for the type."""
+    path = str(tmp_path / "odd_empty.safetensors")
+    write_raw(path, [("u", "U8", [3], bytes([1, 2, 3])), ("e32", "F32", [0, 5], b""), ("e64", "I64", [0], b""),
+                     ("h", "F16", [2], np.array([1.5, -2.0], dtype=np.float16).tobytes()),
+                     ("tail", "BF16", [4, 0], b"")])
+    for layout in ("direct", "window"):
+        loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=2, layout=layout)
+        loader.add_filenames({0: [path]})
+        bufs = loader.copy_files_to_device()
+        assert bufs.get_tensor("u").tolist() == [1, 2, 3]
+        assert bufs.get_tensor("h").tolist() == [1.5, -2.0] and bufs.get_tensor("h").data_ptr() % 16 == 0
+        for name, shape, dt in (("e32", (0, 5), torch.float32), ("e64", (0,), torch.int64), ("tail", (4, 0), torch.bfloat16)):
+            t = bufs.get_tensor(name)
+            assert tuple(t.shape) == shape and t.dtype == dt and t.is_cuda
+        bufs.close()
+        loader.close()
+    assert_clean()
+
+
+@pytest.mark.parametrize("layout", ["direct", "window"])
+def test_downcast_of_types_the_kernel_has_no_pair_for(tmp_path, layout):
+    """Integer tensors next to float weights, and fp8 sources: converted on the GPU by torch's
+    own copy, as the reference converts every tensor (common.py:355-375) -- also when the
+    tensor sits at an offset that is odd for its type."""
+    g = torch.Generator().manual_seed(4)
+    ids = torch.randint(-1000, 1000, (37,), generator=g, dtype=torch.int64)
+    i32 = torch.randint(-70000, 70000, (5, 9), generator=g, dtype=torch.int32)
+    w = torch.randn(33, 17, generator=g) * 3
+    d = torch.randn(11, generator=g, dtype=torch.float64)
+    path = str(tmp_path / "mixed_ints.safetensors")
+    write_raw(path, [("lead", "BF16", [3], torch.ones(3, dtype=torch.bfloat16).view(torch.int16).numpy().tobytes()),
+                     ("ids", "I64", [37], ids.numpy().tobytes()), ("i32", "I32", [5, 9], i32.numpy().tobytes()),
+                     ("w", "F32", [33, 17], w.numpy().tobytes()), ("d", "F64", [11], d.numpy().tobytes())], pad_to=1)
+    ref = {"lead": torch.ones(3, dtype=torch.bfloat16), "ids": ids, "i32": i32, "w": w, "d": d}
+    loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=2, layout=layout)
+    loader.add_filenames({0: [path]})
+    bufs = loader.copy_files_to_device(dtype=DType.BF16)
+    for k, t in ref.items():
+        got = bufs.get_tensor(k)
+        assert got.dtype == torch.bfloat16 and got.shape == t.shape and got.data_ptr() % 16 == 0, k
+        assert torch.equal(got.view(torch.int16).cpu(), t.to(DEV).to(torch.bfloat16).view(torch.int16).cpu()), k
+    bufs.close()
+    # one-byte sources towards fp8: same size, allowed; fp8 -> fp8 and int8 -> fp8 are torch's
+    e5 = (torch.randn(50, generator=g) * 4).to(torch.float8_e5m2)
+    i8 = torch.randint(-100, 100, (21,), generator=g, dtype=torch.int8)
+    h = torch.randn(13, 3, generator=g, dtype=torch.float16)
+    path8 = str(tmp_path / "mixed_fp8.safetensors")
+    write_raw(path8, [("u", "U8", [3], bytes([7, 8, 9])), ("e5", "F8_E5M2", [50], e5.view(torch.uint8).numpy().tobytes()),
+                      ("i8", "I8", [21], i8.numpy().tobytes()), ("h", "F16", [13, 3], h.numpy().tobytes())], pad_to=1)
+    ref8 = {"u": torch.tensor([7, 8, 9], dtype=torch.uint8), "e5": e5, "i8": i8, "h": h}
+    loader.reset()
+    loader.add_filenames({0: [path8]})
+    bufs = loader.copy_files_to_device(dtype=DType.F8_E4M3)
+    for k, t in ref8.items():
+        got = bufs.get_tensor(k)
+        assert got.dtype == torch.float8_e4m3fn and got.shape == t.shape, k
+        assert torch.equal(got.view(torch.uint8).cpu(), t.to(DEV).to(torch.float8_e4m3fn).view(torch.uint8).cpu()), k
+    bufs.close()
+    loader.close()
+    assert_clean()
