@@ -11,10 +11,10 @@
 //   * every request is cut into blocks of `block_bytes` on 4 KiB file
 //     boundaries; workers pull blocks from one FIFO, so a single large file
 //     is read by all workers at once;
-//   * each worker cycles through its own slots of a pinned ring (every worker
-//     allocates its slots itself, once, after binding to the node, so the ring
-//     is placed without touching the creating thread's memory policy and the
-//     sixteen allocations run side by side); after the read it enqueues an asynchronous
+//   * each worker cycles through its own slots of a pinned ring that is
+//     allocated once per context (by a short-lived thread bound to the node, so
+//     the creating thread's affinity and memory policy are never touched);
+//     after the read it enqueues an asynchronous
 //     host-to-device copy and an event on one of the shared copy streams and
 //     moves on to its next slot, so the copy of block k overlaps the read of
 //     block k+1 (the event is waited only when the slot comes round again);
@@ -245,7 +245,7 @@ struct fstx_ctx {
     fstx_config cfg{};
     uint64_t ring_bytes = 0;
     uint64_t slot_bytes = 0;
-    std::vector<char *> rings; // one pinned allocation per worker, made by the worker
+    char *ring = nullptr;
     std::vector<fstx_dev::stream_t> streams;
     std::vector<std::vector<Slot>> slots; // [thread][slot]
     std::vector<std::thread> workers;
@@ -582,19 +582,13 @@ struct Worker {
         ctx->q_cv.notify_all();
     }
 
-    // The worker's share of the pinned ring and its events, made by the worker itself: it is
-    // bound to the node by then, so the memory is placed there without changing the policy of
-    // the thread that creates the context, and the workers allocate side by side.
+    // the worker's share of the ring and the events that guard its slots
     int make_slots() {
-        void *p = nullptr;
-        int rc = fstx_dev::host_alloc(&p, ctx->slot_bytes * ctx->cfg.slots_per_thread);
-        if (rc < 0) return rc;
-        ctx->rings[index] = static_cast<char *>(p);
-        fstx_internal::note_bounce_bytes((int64_t)(ctx->slot_bytes * ctx->cfg.slots_per_thread));
         for (uint32_t k = 0; k < ctx->cfg.slots_per_thread; ++k) {
             Slot s;
-            s.host = ctx->rings[index] + k * ctx->slot_bytes;
-            if ((rc = fstx_dev::event_create(&s.ev)) < 0) return rc;
+            s.host = ctx->ring + ((uint64_t)index * ctx->cfg.slots_per_thread + k) * ctx->slot_bytes;
+            int rc = fstx_dev::event_create(&s.ev);
+            if (rc < 0) return rc;
             mine->push_back(s);
         }
         return 0;
@@ -826,11 +820,10 @@ void free_parts(fstx_ctx *ctx) {
             if (s.ev) fstx_dev::event_destroy(s.ev);
     if (ctx->order_event) fstx_dev::event_destroy(ctx->order_event);
     for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
-    for (char *r : ctx->rings)
-        if (r) {
-            fstx_dev::host_free(r);
-            fstx_internal::note_bounce_bytes(-(int64_t)(ctx->slot_bytes * ctx->cfg.slots_per_thread));
-        }
+    if (ctx->ring) {
+        fstx_dev::host_free(ctx->ring);
+        fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
+    }
 }
 
 void stop_workers(fstx_ctx *ctx) {
@@ -890,8 +883,22 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
     ctx->slot_bytes = cfg.block_bytes + kPage;
     ctx->ring_bytes = ctx->slot_bytes * cfg.n_threads * cfg.slots_per_thread;
-    ctx->rings.assign(cfg.n_threads, nullptr);
     ctx->slots.resize(cfg.n_threads);
+    {
+        // One allocation (sixteen small ones take ten times as long), made by a thread of its
+        // own that binds itself to the node first: the ring is placed there and the caller's
+        // affinity and memory policy stay as they are.
+        void *p = nullptr;
+        std::thread placer([&] {
+            bind_thread_to_node(cfg.numa_node);
+            rc = fstx_dev::set_device(cfg.device_id);
+            if (rc == 0) rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
+        });
+        placer.join();
+        if (rc < 0) return rc;
+        ctx->ring = static_cast<char *>(p);
+        fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
+    }
     for (uint32_t i = 0; i < cfg.n_streams && rc == 0; ++i) {
         fstx_dev::stream_t s = nullptr;
         if ((rc = fstx_dev::stream_create(&s)) == 0) ctx->streams.push_back(s);
