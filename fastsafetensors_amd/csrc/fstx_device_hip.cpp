@@ -113,8 +113,8 @@ int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stre
 
 namespace fstx_internal {
 int check_launch(const char *what) { return rc(hipGetLastError(), what); }
-bool lds_path_disabled() {
-    const char *e = getenv("FSTX_NO_LDS_SLICE"); // read per call so that a benchmark can flip it
-    return e && e[0] == '1';
+int gather_mode() {
+    const char *e = getenv("FSTX_GATHER_MODE"); // read per call so that a benchmark can flip it
+    return e && e[0] >= '0' && e[0] <= '2' ? e[0] - '0' : 1;
 }
 } // namespace fstx_internal

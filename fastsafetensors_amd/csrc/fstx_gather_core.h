@@ -1,0 +1,310 @@
+// SPDX-License-Identifier: Apache-2.0
+//
+// Lane logic of the gather kernel, written against a small memory interface so that the very
+// same code runs per lane on the GPU (fstx_kernels.hip) and per simulated lane on the CPU,
+// where every access is checked against the ranges it may touch (tests/kernel_sim).  No
+// wavefront intrinsics in here: a lane depends on nothing but its tile index, its lane index
+// and the tables, and everything that is derived from the tile index alone is uniform across
+// the wavefront (the compiler keeps it in scalar registers and fetches the tables with scalar
+// loads).
+//
+// The job.  A destination of `rows` rows, `dst_pitch` bytes apart, each holding `row_bytes`
+// payload bytes: the segments of `nsrc` sources side by side, source k contributing `seg`
+// bytes per row at column `col`, read from `src + row * pitch`.  One source and
+// dst_pitch == row_bytes is a rank's block of one tensor (slice extract); several sources are
+// the rank's blocks of several tensors joined along an inner dimension.  Nothing has to be
+// aligned: not the destination, not the pitches, not the segment lengths.
+//
+// How it moves.  The destination is cut into the 16-byte vectors of its memory (vector j is
+// the 16 aligned bytes at align_down(dst, 16) + 16 j); a lane owns one vector: it finds the
+// row and column of the vector's first byte with one 32-bit division, fetches the sixteen
+// bytes with ONE load at whatever byte address they have -- the hardware serves 16-byte global
+// loads at any alignment, measured at the rate of aligned ones -- and writes them with one
+// aligned 16-byte store.  Only the vectors at the seams (a segment ends inside the vector, a
+// pitched destination has a gap there, the job begins or ends there) take the slow way: up to
+// two loads that stay inside their segments, moved into place and blended in registers, and a
+// byte-wise store under a mask when part of the vector is not the job's.  A wavefront thus
+// reads about 1 KiB and writes 1 KiB of contiguous memory whatever the shape; no LDS, no
+// barrier, one pass.
+#ifndef FSTX_GATHER_CORE_H
+#define FSTX_GATHER_CORE_H
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define FSTX_HD __host__ __device__ __forceinline__
+#define FSTX_UNROLL _Pragma("unroll")
+#else
+#define FSTX_HD inline
+#define FSTX_UNROLL
+#endif
+
+namespace fstx_gather {
+
+struct Vec16 {
+    uint32_t w[4];
+};
+
+// 64 bytes: fetched with one wide scalar load.  The job's first source travels inside it, so a
+// job with one source (a slice extract) needs no second, dependent load before its data loads.
+struct alignas(64) Job {
+    char *dst;          // payload byte 0 of row 0, any alignment
+    uint32_t dst_pitch; // bytes between destination rows, >= row_bytes
+    uint32_t row_bytes; // payload bytes per row = sum of the sources' seg
+    uint32_t rows;
+    uint16_t more0;     // sources 1 .. nsrc-1 are more[more0 .. more0 + nsrc - 1) of the launch
+    uint16_t nsrc;
+    uint32_t nvec;      // vectors covering [align_down(dst, 16), last payload byte]
+    uint32_t equal_seg; // != 0: every source has this seg, so column c belongs to source c / seg
+    const char *src;    // source 0: first byte of the block in row 0
+    uint64_t pitch;     //           bytes between its rows
+    uint32_t seg;       //           bytes per row, >= kMinSeg (its column is 0)
+    uint32_t by_die;    // != 0: neighbouring tiles share cache lines (something is not a multiple of 128 bytes)
+    uint64_t pad1;
+};
+
+struct alignas(32) Src {
+    const char *src; // first byte of the block in row 0
+    uint64_t pitch;  // bytes between rows of the source
+    uint32_t seg;    // bytes per row, >= kMinSeg
+    uint32_t col;    // byte offset of the block within a destination row
+    uint64_t pad;
+};
+
+constexpr uint32_t kLanes = 64;
+constexpr uint32_t kVec = 16;
+constexpr uint32_t kTile = kLanes * kVec; // destination bytes per wavefront
+constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two segments
+
+// bytes [m, m + 16) of the 32 bytes lo:hi, m in 0..15.  Written with 64-bit shifts and two-way
+// selects only: a chain of four-way selects over the eight dwords is turned back into an
+// indexed array by the compiler, and that array lands in scratch memory.
+FSTX_HD Vec16 window(Vec16 lo, Vec16 hi, uint32_t m) {
+    const uint64_t p0 = lo.w[0] | (uint64_t)lo.w[1] << 32, p1 = lo.w[2] | (uint64_t)lo.w[3] << 32;
+    const uint64_t p2 = hi.w[0] | (uint64_t)hi.w[1] << 32, p3 = hi.w[2] | (uint64_t)hi.w[3] << 32;
+    const bool far = m >= 8;
+    const uint64_t a0 = far ? p1 : p0, a1 = far ? p2 : p1, a2 = far ? p3 : p2;
+    const uint32_t t = 8 * (m & 7); // 0..56 bits
+    const uint64_t r0 = (a0 >> t) | ((a1 << 1) << (63 - t));
+    const uint64_t r1 = (a1 >> t) | ((a2 << 1) << (63 - t));
+    return Vec16{{(uint32_t)r0, (uint32_t)(r0 >> 32), (uint32_t)r1, (uint32_t)(r1 >> 32)}};
+}
+
+// bytes [at, at + take) from b, the rest from a
+FSTX_HD Vec16 blend(Vec16 a, Vec16 b, uint32_t at, uint32_t take) {
+    Vec16 o;
+    FSTX_UNROLL
+    for (int i = 0; i < 4; ++i) {
+        const int lo = (int)at - 4 * i, hi = (int)(at + take) - 4 * i; // byte range within this dword, unclipped
+        const uint32_t below = lo <= 0 ? 0u : lo >= 4 ? 0xffffffffu : (1u << (8 * lo)) - 1u;   // bytes before the range
+        const uint32_t upto = hi <= 0 ? 0u : hi >= 4 ? 0xffffffffu : (1u << (8 * hi)) - 1u;    // bytes before its end
+        const uint32_t m = upto & ~below;
+        o.w[i] = (a.w[i] & ~m) | (b.w[i] & m);
+    }
+    return o;
+}
+
+// v moved by d bytes, d in -15..15: out[i] = v[i - d]; bytes that come from outside v are zero
+FSTX_HD Vec16 shifted(Vec16 v, int32_t d) {
+    const Vec16 zero = {{0, 0, 0, 0}};
+    const bool up = d > 0;
+    Vec16 lo, hi;
+    FSTX_UNROLL
+    for (int i = 0; i < 4; ++i) {
+        lo.w[i] = up ? 0u : v.w[i];
+        hi.w[i] = up ? v.w[i] : 0u;
+    }
+    (void)zero;
+    return window(lo, hi, up ? kVec - (uint32_t)d : (uint32_t)(-d));
+}
+
+// a segment as one lane sees it
+struct Piece {
+    uint32_t col, len;  // its column within a destination row, its bytes
+    const char *bytes;  // its first byte in the source, in the lane's row
+    const char *lo, *hi; // the source block's readable range: first byte of its first row, one past the last byte of its last row
+};
+
+FSTX_HD Piece piece_from(const char *src, uint64_t pitch, uint32_t seg, uint32_t col, uint32_t row, uint32_t rows) {
+    return Piece{col, seg, src + (uint64_t)row * pitch, src, src + (uint64_t)(rows - 1) * pitch + seg};
+}
+
+// table entry `index`; the index is uniform across the wavefront, so on the GPU these are scalar loads
+FSTX_HD Src src_uniform(const Src *more, uint32_t index) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef uint32_t v8u_ __attribute__((ext_vector_type(8)));
+    const v8u_ raw = *reinterpret_cast<const v8u_ *>(&more[__builtin_amdgcn_readfirstlane(index)]);
+    Src out;
+    __builtin_memcpy(&out, &raw, sizeof out);
+    return out;
+#else
+    return more[index];
+#endif
+}
+
+// which source holds column c of a row (c < row_bytes): the table is read with scalar loads,
+// the comparisons are per lane
+FSTX_HD uint32_t source_of(const Job &jb, const Src *more, uint32_t c) {
+    if (jb.nsrc == 1) return 0;
+    if (jb.equal_seg) return c / jb.equal_seg;
+    uint32_t k = 0;
+    for (uint32_t i = 1; i < jb.nsrc; ++i) k += c >= src_uniform(more, jb.more0 + i - 1).col ? 1u : 0u;
+    return k;
+}
+
+// the first two segments that reach into a tile, worked out once per wavefront with scalar loads
+struct Near {
+    Piece a, b;
+    uint32_t row_a, row_b;
+};
+
+// The segment that holds column c of row `row`.  Nearly every lane lies in one of the two
+// segments at the start of its tile (always, when no segment is shorter than a tile) and takes
+// the description from there; only lanes beyond them look their own up.
+template <bool kMulti>
+FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c, const Near &near) {
+    if (!kMulti || jb.nsrc == 1) return piece_from(jb.src, jb.pitch, jb.seg, 0, row, jb.rows);
+    if (row == near.row_a && c >= near.a.col && c - near.a.col < near.a.len) return near.a;
+    if (row == near.row_b && c >= near.b.col && c - near.b.col < near.b.len) return near.b;
+    const uint32_t k = source_of(jb, more, c);
+    if (k == 0) return piece_from(jb.src, jb.pitch, jb.seg, 0, row, jb.rows);
+    const Src s = more[jb.more0 + k - 1]; // per lane
+    return piece_from(s.src, s.pitch, s.seg, s.col, row, jb.rows);
+}
+
+// One lane's work: vector `lane` of tile `tile` of job `jb`.
+//
+// A vector holds at most two parts (every segment is at least as long as a vector): the rest
+// of the segment in which its first payload byte lies and, when that ends inside the vector,
+// the beginning of the segment that follows -- in the same row, or in the next row behind the
+// gap of a pitched destination.  The addresses of both parts are worked out first, then both
+// loads are issued, and only then is either result looked at: a wavefront that contains a seam
+// waits for memory once, like any other.  A load may reach up to 15 bytes beyond its segment on
+// either side, into the neighbouring bytes of the source block (which the caller guarantees to
+// be readable from the first segment's first byte to the last segment's last byte); at the two
+// ends of the block it is pulled back inside and its result moved into place.
+//
+// kMulti: some job of the launch has more than one source; kPitched: some job's destination rows
+// are further apart than their payload.  A launch without either (rank blocks of single tensors
+// into dense destinations, the common case) runs the lean variant.
+template <bool kMulti, bool kPitched, class Mem>
+FSTX_HD void gather_lane(const Job &jb, const Src *more, uint32_t tile, uint32_t lane, Mem &mem) {
+    const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
+    const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
+    // ---- once per wavefront (joins only): the segment at the start of the tile and the one after it
+    Near near = {{0, 0, nullptr, nullptr, nullptr}, {0, 0, nullptr, nullptr, nullptr}, 0, 0};
+    if (kMulti && jb.nsrc > 1) {
+        const uint32_t t_lo = tile == 0 ? 0u : tile * kTile - head;
+        near.row_a = t_lo / dst_pitch;
+        uint32_t c0 = t_lo - near.row_a * dst_pitch;
+        if (kPitched && c0 >= jb.row_bytes) { // the tile begins in a gap: the next row's first segment
+            c0 = 0;
+            ++near.row_a;
+        }
+        const uint32_t k = source_of(jb, more, c0);
+        const uint32_t k2 = k + 1 < jb.nsrc ? k + 1 : 0u;
+        near.row_b = k2 ? near.row_a : near.row_a + 1;
+        // both descriptions are fetched before either is used (source 0 travels in the job)
+        const Src sa = src_uniform(more, jb.more0 + (k ? k : 1u) - 1);
+        const Src sb = src_uniform(more, jb.more0 + (k2 ? k2 : 1u) - 1);
+        near.a = k ? piece_from(sa.src, sa.pitch, sa.seg, sa.col, near.row_a, jb.rows)
+                   : piece_from(jb.src, jb.pitch, jb.seg, 0, near.row_a, jb.rows);
+        near.b = k2 ? piece_from(sb.src, sb.pitch, sb.seg, sb.col, near.row_b, jb.rows)
+                    : piece_from(jb.src, jb.pitch, jb.seg, 0, near.row_b, jb.rows);
+    }
+    // ---- per lane
+    const uint32_t j = tile * kLanes + lane;
+    if (j >= jb.nvec) return;
+    char *out = jb.dst - head + (uint64_t)kVec * j;
+    // pitched position p is destination byte dst + p: row p / dst_pitch, column p % dst_pitch
+    uint32_t at = j == 0 ? head : 0u;       // vector 0 begins `head` bytes before the job does
+    const uint32_t q = kVec * j - head;     // position of the vector's byte 0 (wraps for j == 0 when head > 0)
+    uint32_t row = (q + at) / dst_pitch;
+    uint32_t c = (q + at) - row * dst_pitch;
+    if (kPitched && c >= jb.row_bytes) { // the vector begins in the gap behind a row's payload
+        at += dst_pitch - c;
+        c = 0;
+        ++row;
+    }
+    if (at >= kVec || row >= jb.rows) return; // nothing of the job in this vector
+    // ---- part 1
+    const Piece p1 = piece_of<kMulti>(jb, more, row, c, near);
+    const uint32_t in1 = c - p1.col;
+    const uint32_t at1 = at;
+    const uint32_t take1 = p1.len - in1 < kVec - at1 ? p1.len - in1 : kVec - at1;
+    const char *ideal1 = p1.bytes + in1 - at1; // where a load has to start to put the segment's byte in1 at byte at1
+    const char *addr1 = ideal1 < p1.lo ? p1.lo : ideal1 + kVec > p1.hi ? p1.hi - kVec : ideal1;
+    // ---- part 2
+    uint32_t at2 = at1 + take1, c2 = c + take1, row2 = row;
+    if (c2 == jb.row_bytes) { // the row's payload ends: over the gap (if any) into the next row
+        if (kPitched) at2 += dst_pitch - jb.row_bytes;
+        c2 = 0;
+        ++row2;
+    }
+    const bool has2 = at2 < kVec && row2 < jb.rows;
+    Vec16 g2 = {{0, 0, 0, 0}};
+    const char *ideal2 = nullptr, *addr2 = nullptr;
+    if (has2) {
+        const Piece p2 = piece_of<kMulti>(jb, more, row2, c2, near); // c2 is a segment's first column
+        ideal2 = p2.bytes - at2;
+        addr2 = ideal2 < p2.lo ? p2.lo : ideal2; // (the vector ends inside the segment: it is at least a vector long)
+    }
+    // ---- both loads, then the arithmetic
+    Vec16 g1 = mem.load16_stream(addr1);
+    if (has2) g2 = mem.load16(addr2);
+    const uint32_t from2 = has2 ? at2 : kVec; // bytes [from2, 16) come from part 2
+    const bool plain = at1 == 0 && at1 + take1 >= from2 && addr1 == ideal1 && (!has2 || addr2 == ideal2);
+    if (plain) {
+        // nearly every vector, seams between segments included: straight-line code for the whole wavefront
+        mem.store16(out, blend(g1, g2, from2, kVec - from2));
+        return;
+    }
+    // the rest: the two ends of a source block (the load was pulled back inside it) and vectors
+    // that are only partly the job's (its two ends, the gaps of a pitched destination)
+    if (addr1 != ideal1) g1 = shifted(g1, (int32_t)(addr1 - ideal1));
+    uint32_t mask = ((1u << take1) - 1u) << at1; // bit i: byte i of the vector is payload
+    Vec16 acc = g1;
+    if (has2) {
+        if (addr2 != ideal2) g2 = shifted(g2, (int32_t)(addr2 - ideal2));
+        acc = blend(acc, g2, at2, kVec - at2);
+        mask |= 0xffffu & (0xffffu << at2);
+    }
+    if (mask == 0xffffu) {
+        mem.store16(out, acc);
+    } else {
+        FSTX_UNROLL
+        for (uint32_t i = 0; i < kVec; ++i)
+            if (mask >> i & 1u) mem.store8(out + i, (unsigned char)(acc.w[i >> 2] >> (8 * (i & 3))));
+    }
+}
+
+// ---- host side: the shapes the kernel takes, and how a job is cut to fit 32-bit positions
+
+// Positions (bytes counted from the job's first, rows dst_pitch apart) are 32-bit in the kernel;
+// a job may span this many at most, which leaves room for the tile that holds the last one.
+constexpr uint64_t kMaxSpan = 0xffffffffull - 2 * kTile;
+
+inline bool shape_ok(uint64_t dst_pitch, uint64_t row_bytes, uint64_t min_seg) {
+    return min_seg >= kMinSeg && row_bytes <= dst_pitch && dst_pitch <= kMaxSpan;
+}
+
+// rows one job may cover (>= 1 when shape_ok)
+inline uint64_t rows_per_job(uint64_t dst_pitch, uint64_t row_bytes) {
+    return (kMaxSpan - row_bytes) / dst_pitch + 1;
+}
+
+// `first` is the job's source 0 (its col is 0); sources 1 .. nsrc-1 sit at more[more0 ..] of the launch
+inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t rows, const Src &first, uint32_t more0,
+                    uint32_t nsrc, uint64_t equal_seg, bool by_die = true) {
+    const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
+    const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
+    return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,
+               (uint32_t)((head + span + kVec - 1) / kVec), (uint32_t)equal_seg, first.src, first.pitch, first.seg,
+               by_die ? 1u : 0u, 0};
+}
+
+inline uint64_t tiles_of(const Job &jb) { return ((uint64_t)jb.nvec + kLanes - 1) / kLanes; }
+
+} // namespace fstx_gather
+
+#endif

@@ -40,7 +40,10 @@ int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stre
 namespace fstx_internal {
 
 int check_launch(const char *what);  // hipGetLastError -> 0 / -FSTX_E_HIP
-bool lds_path_disabled();            // FSTX_NO_LDS_SLICE=1: odd-aligned slices stay on the direct kernel (measurements)
+// FSTX_GATHER_MODE, for measurements: 0 the gather kernel is never used (unit-sized moves instead),
+// 1 (default) it serves every strided shape but dense cuts that are 16-byte aligned throughout,
+// 2 those too
+int gather_mode();
 bool debug_enabled();
 void debug(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 void note_bounce_bytes(int64_t delta); // process-wide pinned ring accounting

@@ -9,9 +9,12 @@
 //                    (cpp/ext.cpp:606-645: two cudaMemcpy through a temporary).
 //   slice extract  : dense copy of `outer` segments read at a fixed pitch.
 //                    Stands in for t[slices].contiguous() per rank in
-//                    LazyTensorFactory.shuffle (tensor_factory.py:168-175).
-//                    Three forms: direct, strided destination (joins), and
-//                    staged through LDS for shapes that are not 16-byte multiples.
+//                    LazyTensorFactory.shuffle (tensor_factory.py:168-175), and, with
+//                    several sources side by side, for that plus torch.cat in
+//                    shuffle_multi_cols (tensor_factory.py:194-259).  The gather kernel
+//                    serves every shape and alignment with 16-byte loads at the data's own
+//                    byte address; a 16-byte-unit kernel serves cuts that are aligned
+//                    throughout, a small-unit kernel segments shorter than 16 bytes.
 //   down-cast      : element type conversion towards a narrower type with torch's
 //                    rounding (SafeTensorsMetadata.get_tensors with a dtype,
 //                    common.py:355-375).
@@ -19,14 +22,15 @@
 // Every kernel takes a table of jobs as a by-value kernel argument (up to
 // FSTX_BATCH_MAX), so that the many small tensors of a checkpoint file cost one
 // launch.  A workgroup is one wavefront and owns 64 consecutive 16-byte vectors
-// of one job's destination (a 2 KiB tile in the LDS form); consecutive lanes touch
-// consecutive vectors, so each wavefront reads and writes contiguous spans.
+// of one job's destination; consecutive lanes touch consecutive vectors, so each
+// wavefront reads and writes contiguous spans.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
 
 #include "fstx.h"
+#include "fstx_gather_core.h"
 #include "fstx_internal.h"
 
 namespace {
@@ -86,13 +90,15 @@ typedef uint32_t v16u __attribute__((ext_vector_type(16)));
 
 // Kernel arguments are limited to 4 KiB: 48 jobs of 32 bytes or 24 jobs of 64 bytes fit
 // next to the two lookup tables.
-template <typename Job>
+template <typename Job, uint32_t kJobsN = (sizeof(Job) == 32 ? FSTX_BATCH_MAX : FSTX_BATCH_MAX / 2),
+          uint32_t kSlotsN = kOwnerSlots>
 struct JobTable {
     static_assert(sizeof(Job) == 32 || sizeof(Job) == 64, "jobs are fetched as eight or sixteen dwords");
-    static constexpr uint32_t kJobs = sizeof(Job) == 32 ? FSTX_BATCH_MAX : FSTX_BATCH_MAX / 2;
+    static constexpr uint32_t kJobs = kJobsN;
+    static constexpr uint32_t kSlots = kSlotsN;
     Job job[kJobs];
-    uint32_t first_block[kJobs];     // first workgroup of each job (granule aligned)
-    uint32_t owner[kOwnerSlots / 4]; // one byte per granule: index into job[]
+    uint32_t first_block[kJobs]; // first workgroup of each job (granule aligned)
+    uint32_t owner[kSlots / 4];  // one byte per granule: index into job[]
 
     // the whole job in one scalar load
     __device__ __forceinline__ Job fetch(uint32_t ji) const {
@@ -108,20 +114,20 @@ struct JobTable {
     }
 };
 
-template <typename Job>
-__device__ __forceinline__ uint32_t find_job(const JobTable<Job> &t, uint32_t granule_log2, uint32_t b) {
+template <typename Table>
+__device__ __forceinline__ uint32_t find_job(const Table &t, uint32_t granule_log2, uint32_t b) {
     const uint32_t g = b >> granule_log2;
     return (t.owner[g >> 2] >> ((g & 3) * 8)) & 0xffu;
 }
 
 // Host side: lays the jobs' workgroup counts out on granules; returns the grid size.
-template <typename Job>
-inline uint64_t plan_grid(JobTable<Job> &t, const uint64_t *blocks_of, uint32_t n, uint32_t *granule_log2) {
+template <typename Table>
+inline uint64_t plan_grid(Table &t, const uint64_t *blocks_of, uint32_t n, uint32_t *granule_log2) {
     uint32_t gl = 0;
     for (;; ++gl) {
         uint64_t need = 0;
         for (uint32_t i = 0; i < n; ++i) need += (blocks_of[i] + (1ull << gl) - 1) >> gl;
-        if (need <= kOwnerSlots) break;
+        if (need <= Table::kSlots) break;
     }
     uint64_t granule = 0;
     uint8_t *owner = reinterpret_cast<uint8_t *>(t.owner);
@@ -313,246 +319,57 @@ __global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t granule_
     }
 }
 
-// Fused slice + concatenate along an inner dimension.  The destination is swept in row
-// order: a chunk is `rows_per_chunk` rows of the joined tensor, and within a chunk the
-// sources follow one another, each with whole wavefronts of its own (a wavefront never
-// mixes sources, so everything that selects the source is scalar work).  Writes therefore
-// stay within a few hundred KB of one another instead of striding through the whole
-// destination once per source.
-struct alignas(32) JoinSrc {
-    const char *src;     // the block's first byte in row 0
-    uint64_t src_pitch;
-    uint32_t seg_units;  // units per row
-    uint32_t dst_col;    // byte offset of the block in a joined row
-    uint64_t pad;
-};
-
-struct JoinTable {
-    char *dst;
-    uint64_t dst_pitch;       // bytes of a joined row
-    uint32_t rows, rows_per_chunk, waves_per_chunk, n, unit_log2;
-    uint32_t wave_begin[FSTX_JOIN_MAX]; // first wavefront of each source within a chunk
-    JoinSrc src[FSTX_JOIN_MAX];
-};
-
-template <typename Unit>
-__device__ __forceinline__ void join_units(const JoinTable &t, const JoinSrc &js, uint32_t chunk, uint32_t u) {
-    const uint32_t r = u / js.seg_units;
-    const uint32_t col = u - r * js.seg_units;
-    const uint64_t row = (uint64_t)chunk * t.rows_per_chunk + r;
-    if (r >= t.rows_per_chunk || row >= t.rows) return; // idle lanes at the end of a source's share
-    const Unit *src = reinterpret_cast<const Unit *>(js.src + row * js.src_pitch) + col;
-    Unit *dst = reinterpret_cast<Unit *>(t.dst + row * t.dst_pitch + js.dst_col) + col;
-    st_stream(ld_stream(src), dst);
-}
-
-__global__ __launch_bounds__(kBlock) void join_kernel(const JoinTable t) {
-    const uint32_t b = blockIdx.x;
-    const uint32_t chunk = b / t.waves_per_chunk;
-    const uint32_t w = b - chunk * t.waves_per_chunk;
-    uint32_t k = 0;
-    for (uint32_t j = 1; j < t.n; ++j) k += w >= t.wave_begin[j] ? 1u : 0u; // uniform: scalar compares
-    const v8u raw = *reinterpret_cast<const v8u *>(&t.src[k]);
-    JoinSrc js;
-    __builtin_memcpy(&js, &raw, sizeof js);
-    const uint32_t u = (w - t.wave_begin[k]) * kBlock + threadIdx.x;
-    switch (t.unit_log2) { // uniform across the launch
-    case 4: join_units<v4u>(t, js, chunk, u); break;
-    case 3: join_units<uint64_t>(t, js, chunk, u); break;
-    case 2: join_units<uint32_t>(t, js, chunk, u); break;
-    case 1: join_units<uint16_t>(t, js, chunk, u); break;
-    default: join_units<uint8_t>(t, js, chunk, u); break;
-    }
-}
-
-// ------------------------------------- slice extract, staged through LDS
+// ----------------------------------------------------------------- gather
 //
-// For segments whose length, pitch or source address is not a multiple of 16
-// bytes the direct kernel above has to drop to 8-, 4-, 2- or 1-byte moves per
-// lane.  This variant keeps every global access 16 bytes wide: a wavefront owns
-// a 2 KiB tile of the (16-byte aligned) destination, loads the aligned 16-byte
-// source vectors that cover the tile's rows into LDS -- each row into its own
-// slot, at the same offset modulo 16 it has in memory -- and then reads each
-// destination vector back with one 16-byte LDS read at the byte address where its
-// data begins.  The odd alignment is absorbed by LDS, which serves unaligned reads.
+// Slice extract and fused slice + join for any shape and alignment: the lane logic is in
+// fstx_gather_core.h (it also runs on the CPU under the bounds-checking simulator of the
+// tests).  One 16-byte load at the data's own byte address, one aligned 16-byte store; a
+// launch carries up to FSTX_BATCH_MAX jobs and FSTX_BATCH_MAX sources in its arguments.
 
-#ifndef FSTX_LDS_TILE
-#define FSTX_LDS_TILE 2048
-#endif
-constexpr uint32_t kTileBytes = FSTX_LDS_TILE; // destination bytes per wavefront
-constexpr uint32_t kLdsMinSeg = 64;   // shorter segments stay on the direct kernel
-// LDS slot of the tile's i-th row piece starts at align_down(s_i + 48 i, 16), where s_i is
-// the piece's position in the tile: consecutive slots then never overlap (a piece of L bytes
-// needs at most L + 30 bytes once both ends are widened to 16-byte vectors), and a tile
-// touches at most floor((tile - 2) / seg) + 2 rows.
-constexpr uint32_t kRowGap = 48;
-// LDS a wavefront needs when no segment of the launch is shorter than min_seg: the fewer rows
-// a tile can touch, the less LDS per wavefront and the more wavefronts a CU keeps in flight
-// (3.7 KB at 64-byte segments, 2.3 KB from 2 KiB segments up).  2 KiB tiles measured a
-// little faster than 4 KiB ones (5.5 against 5.3 TB/s), 1 KiB and 8 KiB ones slower.
-inline uint32_t lds_bytes_for(uint64_t min_seg) {
-    const uint32_t rows = (uint32_t)((kTileBytes - 2) / min_seg) + 2;
-    return kTileBytes + kRowGap * (rows + 1) + 64;
-}
+typedef v4u v4u_anywhere __attribute__((aligned(1)));
 
-struct alignas(32) LdsSliceJob {
-    char *dst;            // 16-byte aligned
-    const char *src;
-    uint64_t pitch_unit;  // pitch (< 2^56) | log2(unit bytes) << 56
-    uint32_t seg_bytes;   // kLdsMinSeg <= seg_bytes
-    uint32_t outer;       // number of segments
+struct GatherMem {
+    // the bulk: streaming loads (every byte of a checkpoint is cut once)
+    __device__ __forceinline__ fstx_gather::Vec16 load16_stream(const char *p) {
+        const v4u v = __builtin_nontemporal_load((const FSTX_GLOBAL v4u_anywhere *)p);
+        return fstx_gather::Vec16{{v.x, v.y, v.z, v.w}};
+    }
+    // the seams: plain loads, their cache lines are about to be used by the neighbouring lanes
+    __device__ __forceinline__ fstx_gather::Vec16 load16(const char *p) {
+        const v4u v = *(const FSTX_GLOBAL v4u_anywhere *)p;
+        return fstx_gather::Vec16{{v.x, v.y, v.z, v.w}};
+    }
+    __device__ __forceinline__ void store16(char *p, fstx_gather::Vec16 v) {
+        st_stream(v4u{v.w[0], v.w[1], v.w[2], v.w[3]}, reinterpret_cast<v4u *>(p));
+    }
+    __device__ __forceinline__ void store8(char *p, unsigned char b) { st_global(b, reinterpret_cast<unsigned char *>(p)); }
 };
 
-// Geometry of one tile in 32-bit arithmetic.  Positions are counted in bytes from column 0
-// of the tile's first row: destination byte p of the tile is position first_col + p, local
-// row i covers positions [i * seg, (i + 1) * seg).  seg < 2^31 keeps all of it below 2^32.
-struct TileGeom {
-    uint32_t seg, first_col, end_pos, src_lo, pitch_lo;
-
-    __device__ __forceinline__ uint32_t col_begin(uint32_t i) const { return i == 0 ? first_col : 0u; }
-    // LDS offset of the 16-byte vector that receives the first source vector of row piece i
-    __device__ __forceinline__ uint32_t slot(uint32_t i) const {
-        const uint32_t s = i * seg + col_begin(i) - first_col; // where the piece starts in the tile
-        return (s + kRowGap * i) & ~15u;
-    }
-    // LDS offset of column 0 of local row i (for row 0 it may lie before the slot; the
-    // difference wraps consistently in 32 bits and is only used with col >= col_begin)
-    __device__ __forceinline__ uint32_t row_base(uint32_t i) const {
-        const uint32_t cb = col_begin(i);
-        const uint32_t mis = (src_lo + i * pitch_lo + cb) & 15u; // the piece's source address mod 16
-        return slot(i) + mis - cb;
-    }
+// per launch: 32 jobs (each carries its first source), 24 further sources of joins, 1,024 granules
+constexpr uint32_t kGatherJobs = 32;
+constexpr uint32_t kGatherMore = FSTX_JOIN_MAX;
+struct GatherTable : JobTable<fstx_gather::Job, kGatherJobs, 1024> {
+    fstx_gather::Src more[kGatherMore];
 };
+static_assert(sizeof(GatherTable) + 32 <= 4096, "kernel arguments are limited to 4 KiB");
 
-// 16 bytes of LDS at any byte address (the hardware runs DS operations in unaligned mode)
-typedef v4u lds_vec __attribute__((aligned(1)));
-
-// (Reading five dwords at the dword boundary below and funnel-shifting them measured the same.)
-__device__ __forceinline__ v4u lds_read16(const unsigned char *lds, uint32_t addr) {
-    return *reinterpret_cast<const lds_vec *>(lds + addr);
-}
-
-__device__ __forceinline__ void lds_tile(const LdsSliceJob &job, uint32_t tile, unsigned char *lds) {
-    const uint32_t lane = threadIdx.x;
-    const uint64_t pitch = job.pitch_unit & 0x00ffffffffffffffull;
-    const uint32_t seg = job.seg_bytes;
-    const uint64_t total = (uint64_t)job.outer * seg;
-    const uint64_t d0 = (uint64_t)tile * kTileBytes;
-    const uint32_t tile_bytes = total - d0 < kTileBytes ? (uint32_t)(total - d0) : kTileBytes;
-    // the tile's first row; a 32-bit division whenever the job is smaller than 4 GiB
-    const uint64_t row_first = (total >> 32) == 0 ? (uint64_t)((uint32_t)d0 / seg) : d0 / seg;
-    TileGeom g;
-    g.seg = seg;
-    g.first_col = (uint32_t)(d0 - row_first * seg);
-    g.end_pos = g.first_col + tile_bytes;
-    g.pitch_lo = (uint32_t)pitch;
-    g.src_lo = (uint32_t)(uintptr_t)job.src + (uint32_t)row_first * g.pitch_lo; // low address bits are all that matter
-    const uint32_t nrows = (g.end_pos - 1) / seg + 1;
-    const char *src_row0 = job.src + row_first * pitch;
-
-    // ---- phase 1: aligned 16-byte loads into LDS.  `group` lanes share a row piece; short
-    // rows are loaded several per step so that the lanes stay busy.
-    const uint32_t longest = seg < kTileBytes ? seg : kTileBytes;
-    const uint32_t vmax = (longest + 30) / 16 + 1; // vectors a row piece can need
-    uint32_t group_log2 = 6;
-    while (group_log2 > 0 && (32u >> (6 - group_log2)) >= vmax) --group_log2;
-    const uint32_t group = 1u << group_log2;
-    if (group_log2 == 6) {
-        // Long row pieces, one per step: the loads go from global memory straight into LDS
-        // (lane l of an instruction lands at the instruction's LDS base + 16 l), no register
-        // in between, so all loads of the tile are in flight before the first one is waited for.
-        for (uint32_t i = 0; i < nrows; ++i) {
-            const uint32_t cb = g.col_begin(i);
-            const uint32_t pos_end = (i + 1) * seg < g.end_pos ? (i + 1) * seg : g.end_pos;
-            const uintptr_t a0 = (uintptr_t)src_row0 + (uint64_t)i * pitch + cb;
-            const uintptr_t a1 = a0 + (pos_end - (i * seg + cb));
-            const uintptr_t lo = a0 & ~(uintptr_t)15;
-            const uint32_t at = g.slot(i);
-            for (uint32_t base = 0; lo + 16ull * base < a1; base += 64) {
-                const uintptr_t mine = lo + 16ull * (base + lane);
-                if (mine < a1)
-                    __builtin_amdgcn_global_load_lds((const FSTX_GLOBAL void *)mine,
-                                                     (__attribute__((address_space(3))) void *)(lds + at + 16 * base),
-                                                     16, 0, 0);
-            }
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    } else {
-        for (uint32_t ibase = 0; ibase < nrows; ibase += 64u >> group_log2) {
-            const uint32_t i = ibase + (lane >> group_log2);
-            if (i < nrows) {
-                const uint32_t cb = g.col_begin(i);
-                const uint32_t pos_end = (i + 1) * seg < g.end_pos ? (i + 1) * seg : g.end_pos;
-                const uintptr_t a0 = (uintptr_t)src_row0 + (uint64_t)i * pitch + cb;
-                const uintptr_t a1 = a0 + (pos_end - (i * seg + cb));
-                const uintptr_t lo = a0 & ~(uintptr_t)15;
-                const uint32_t at = g.slot(i);
-                // plain loads, not streaming ones: the cache lines at the ends of a piece are shared
-                // with the neighbouring tile, and streaming lines were fetched from HBM again for it
-                // (fetch traffic 9.6 % over the algorithmic bytes against 3.1 % with plain loads)
-                for (uint32_t v = lane & (group - 1); lo + 16ull * v < a1; v += group)
-                    *reinterpret_cast<v4u *>(lds + at + 16 * v) = ld_global(reinterpret_cast<const v4u *>(lo) + v);
-            }
-        }
-    }
-    __syncthreads(); // one wavefront: orders its LDS writes before the reads below
-
-    // ---- phase 2: one 16-byte LDS read per destination vector, at whatever alignment the
-    // source had; a vector that runs over the end of a row takes its remaining bytes from
-    // the start of the next row (rows are at least 64 bytes, so never from a third).
-    for (uint32_t p = 16 * lane; p < tile_bytes; p += 16 * 64) {
-        const uint32_t pos = g.first_col + p;
-        const uint32_t i = pos / seg;
-        const uint32_t col = pos - i * seg;
-        const uint32_t n = tile_bytes - p < 16 ? tile_bytes - p : 16u; // < 16 only at the end of the job
-        const uint32_t in_row = seg - col;
-        v4u out = lds_read16(lds, g.row_base(i) + col);
-        if (in_row < n) {
-            const v4u next = lds_read16(lds, g.row_base(i + 1) - in_row);
-            uint32_t o[4] = {out.x, out.y, out.z, out.w};
-            const uint32_t x[4] = {next.x, next.y, next.z, next.w};
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                // bytes of this dword that still belong to the current row: 0..4
-                const int keep = (int)in_row - 4 * w;
-                const uint32_t m = keep >= 4 ? 0xffffffffu : keep <= 0 ? 0u : (1u << (8 * keep)) - 1u;
-                o[w] = (o[w] & m) | (x[w] & ~m);
-            }
-            out = v4u{o[0], o[1], o[2], o[3]};
-        }
-        char *dst = job.dst + d0 + p;
-        if (n == 16) {
-            st_stream(out, reinterpret_cast<v4u *>(dst));
-        } else { // the job's last, partial vector
-            const uint32_t o[4] = {out.x, out.y, out.z, out.w};
-#pragma unroll
-            for (int q = 0; q < 16; ++q)
-                if ((uint32_t)q < n) st_global((unsigned char)(o[q / 4] >> (8 * (q % 4))), reinterpret_cast<unsigned char *>(dst) + q);
-        }
-    }
-}
-
-__global__ __launch_bounds__(64) void slice_lds_kernel(const uint32_t granule_log2,
-                                                       const JobTable<LdsSliceJob> t) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[]; // lds_bytes_for(shortest segment)
+template <bool kMulti, bool kPitched>
+__global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2, const GatherTable t) {
     const uint32_t b = blockIdx.x;
     const uint32_t ji = find_job(t, granule_log2, b);
-    const LdsSliceJob job = t.fetch(ji);
+    const fstx_gather::Job job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
-    // Neighbouring tiles share the source cache lines that their common border cuts through.
-    // Workgroups go round-robin over the eight dies, so give each die one contiguous eighth of
-    // the job's tiles: the shared line is then found in that die's L2 instead of being fetched twice.
-    const uint64_t n_tiles = ((uint64_t)job.outer * job.seg_bytes + kTileBytes - 1) / kTileBytes;
-    const uint32_t per_die = (uint32_t)((n_tiles + kXcds - 1) / kXcds);
-#ifdef FSTX_LDS_NO_XCD_MAP
-    const uint32_t tile = lb;
-    if (tile >= n_tiles) return;
-#else
+    // neighbouring tiles share the cache lines their common border cuts through: one contiguous
+    // eighth of the job per die (workgroup b runs on die b % 8), so that the shared line is found
+    // in that die's L2 and a destination line is completed within one L2
+    // (in dispatch order when everything sits on cache-line boundaries and nothing is shared)
+    const uint32_t n_tiles = (job.nvec + fstx_gather::kLanes - 1) / fstx_gather::kLanes;
+    const uint32_t per_die = (n_tiles + kXcds - 1) / kXcds;
     const uint32_t turn = lb / kXcds;
-    const uint32_t tile = (lb % kXcds) * per_die + turn;
-    if (turn >= per_die || tile >= n_tiles) return; // idle padding of the last eighth and granule
-#endif
-    lds_tile(job, tile, lds);
+    const uint32_t tile = job.by_die ? (lb % kXcds) * per_die + turn : lb;
+    if ((job.by_die && turn >= per_die) || tile >= n_tiles) return; // idle padding of the last eighth and granule
+    GatherMem mem;
+    fstx_gather::gather_lane<kMulti, kPitched>(job, t.more, tile, threadIdx.x, mem);
 }
 
 // ------------------------------------------------- down-cast while loading
@@ -744,6 +561,99 @@ inline Limits limits() {
 }
 inline bool grid_fits(uint64_t workgroups) { return workgroups * kBlock <= 0xffffffffull; }
 
+// Collects gather jobs and their sources for launches of gather_kernel.
+struct GatherBatch {
+    GatherTable t;
+    uint64_t tiles_of[kGatherJobs];
+    uint64_t tiles = 0;
+    uint32_t nj = 0, ns = 0;
+    bool multi = false, pitched = false; // what the jobs collected so far ask of the kernel
+    hipStream_t stream;
+    Limits lim;
+
+    explicit GatherBatch(void *s) : stream(static_cast<hipStream_t>(s)), lim(limits()) {}
+
+    int flush() {
+        if (nj == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t grid = plan_grid(t, tiles_of, nj, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        // the leanest variant that serves every job of the launch
+        if (multi && pitched) hipLaunchKernelGGL((gather_kernel<true, true>), dim3((uint32_t)grid), dim3(64), 0, stream, gl, t);
+        else if (multi) hipLaunchKernelGGL((gather_kernel<true, false>), dim3((uint32_t)grid), dim3(64), 0, stream, gl, t);
+        else if (pitched) hipLaunchKernelGGL((gather_kernel<false, true>), dim3((uint32_t)grid), dim3(64), 0, stream, gl, t);
+        else hipLaunchKernelGGL((gather_kernel<false, false>), dim3((uint32_t)grid), dim3(64), 0, stream, gl, t);
+        nj = ns = 0;
+        tiles = 0;
+        multi = pitched = false;
+        return fstx_internal::check_launch("gather_kernel");
+    }
+
+    // whether the kernel takes this shape (every segment at least 16 bytes, rows that fit 32-bit positions)
+    static bool takes(uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n) {
+        uint64_t row_bytes = 0, min_seg = ~0ull;
+        uint32_t live = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            if (srcs[i].seg_bytes == 0) continue;
+            row_bytes += srcs[i].seg_bytes;
+            if (srcs[i].seg_bytes < min_seg) min_seg = srcs[i].seg_bytes;
+            if (rows > 1 && srcs[i].src_pitch >> 56) return false;
+            ++live;
+        }
+        if (live == 0 || live > kGatherMore) return false;
+        return fstx_gather::shape_ok(dst_pitch ? dst_pitch : row_bytes, row_bytes, min_seg);
+    }
+
+    // rows x (segments of the n sources side by side) into dst, rows dst_pitch apart (0: dense)
+    int add(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n) {
+        fstx_join_src live[kGatherMore];
+        uint32_t m = 0;
+        uint64_t row_bytes = 0, equal = 0, bits = (uint64_t)(uintptr_t)dst;
+        for (uint32_t i = 0; i < n; ++i) {
+            if (srcs[i].seg_bytes == 0) continue;
+            if (m == 0) equal = srcs[i].seg_bytes;
+            if (srcs[i].seg_bytes != equal) equal = 0;
+            live[m++] = srcs[i];
+            row_bytes += srcs[i].seg_bytes;
+            bits |= (uint64_t)(uintptr_t)srcs[i].src | srcs[i].seg_bytes | srcs[i].src_pitch;
+        }
+        if (dst_pitch == 0) dst_pitch = row_bytes;
+        const bool lines_shared = ((bits | dst_pitch) & 127) != 0;
+        // rows per job: 32-bit positions, and no more tiles than one job may take
+        uint64_t per_job = fstx_gather::rows_per_job(dst_pitch, row_bytes);
+        const uint64_t by_tiles = lim.job * fstx_gather::kTile / dst_pitch;
+        if (by_tiles < per_job) per_job = by_tiles;
+        if (per_job == 0) return -FSTX_E_RANGE; // one row is more than a job holds
+        for (uint64_t row = 0; row < rows; row += per_job) {
+            const uint64_t part = rows - row < per_job ? rows - row : per_job;
+            auto source = [&](uint32_t i, uint64_t col) {
+                return fstx_gather::Src{static_cast<const char *>(live[i].src) + row * live[i].src_pitch, live[i].src_pitch,
+                                        (uint32_t)live[i].seg_bytes, (uint32_t)col, 0};
+            };
+            fstx_gather::Job job = fstx_gather::make_job(static_cast<char *>(dst) + row * dst_pitch, dst_pitch, row_bytes,
+                                                         part, source(0, 0), 0, m, m > 1 ? equal : 0, lines_shared);
+            const uint64_t need = (fstx_gather::tiles_of(job) + kXcds - 1) / kXcds * kXcds; // whole eighths
+            if (nj == kGatherJobs || ns + m - 1 > kGatherMore || tiles + need > lim.launch) {
+                int rc = flush();
+                if (rc < 0) return rc;
+            }
+            job.more0 = (uint16_t)ns;
+            uint64_t col = live[0].seg_bytes;
+            for (uint32_t i = 1; i < m; ++i) {
+                t.more[ns++] = source(i, col);
+                col += live[i].seg_bytes;
+            }
+            t.job[nj] = job;
+            tiles_of[nj] = need;
+            tiles += need;
+            ++nj;
+            multi |= m > 1;
+            pitched |= dst_pitch != row_bytes;
+        }
+        return 0;
+    }
+};
+
 } // namespace
 
 extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, void *stream) {
@@ -797,27 +707,21 @@ extern "C" int fstx_realign_copy(void *dst, const void *src, uint64_t nbytes, vo
     return fstx_realign_copy_batch(&d, 1, stream);
 }
 
+// Where a strided cut goes.  Contiguous spans never get here (they go to the realign copy).
+//   gather_kernel   every shape with segments of at least 16 bytes: dense and pitched
+//                   destinations, one source or several, any alignment of anything;
+//   slice_kernel    dense cuts in which every address, segment and pitch is a multiple of 16
+//                   bytes: nothing to realign, 3 % faster than the gather on such shapes;
+//   slice2d_kernel  what is left: segments shorter than 16 bytes (and FSTX_GATHER_MODE=0, for
+//                   measurements), moved in the largest unit of 1..16 bytes that divides everything.
 extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, void *stream) {
     if (n == 0) return 0;
     if (!descs) return -FSTX_E_INVAL;
     if (n > FSTX_BATCH_MAX) return -FSTX_E_TOO_MANY;
     JobTable<SliceJob> t;
-    JobTable<LdsSliceJob> tl;
-    uint64_t blocks_of[FSTX_BATCH_MAX], tiles_of[FSTX_BATCH_MAX];
-    uint64_t blocks = 0, tiles = 0, min_seg = ~0ull;
-    uint32_t k = 0, kl = 0;
-    auto flush_lds = [&]() -> int {
-        if (kl == 0) return 0;
-        uint32_t gl = 0;
-        const uint64_t grid = plan_grid(tl, tiles_of, kl, &gl);
-        if (!grid_fits(grid)) return -FSTX_E_RANGE;
-        hipLaunchKernelGGL(slice_lds_kernel, dim3((uint32_t)grid), dim3(64), lds_bytes_for(min_seg),
-                           static_cast<hipStream_t>(stream), gl, tl);
-        kl = 0;
-        tiles = 0;
-        min_seg = ~0ull;
-        return fstx_internal::check_launch("slice_lds_kernel");
-    };
+    uint64_t blocks_of[FSTX_BATCH_MAX];
+    uint64_t blocks = 0;
+    uint32_t k = 0;
     auto flush = [&]() -> int {
         if (k == 0) return 0;
         uint32_t gl = 0;
@@ -832,6 +736,8 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     fstx_copy_desc spans[FSTX_BATCH_MAX];
     uint32_t n_spans = 0;
     const Limits lim = limits();
+    const int mode = fstx_internal::gather_mode();
+    GatherBatch gather(stream);
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_slice_desc &d = descs[i];
         if (d.outer == 0 || d.seg_bytes == 0) continue;
@@ -846,21 +752,10 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         uint64_t outer = d.outer, seg = d.seg_bytes, pitch = d.src_pitch;
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src |
                                              seg | pitch | 16u);
-        if (ul < 4 && seg >= kLdsMinSeg && seg < 0x80000000ull && outer <= 0xffffffffull &&
-            ((uintptr_t)d.dst & 15) == 0 && (outer * seg + kTileBytes - 1) / kTileBytes + kXcds <= lim.job &&
-            !fstx_internal::lds_path_disabled()) {
-            // odd alignment somewhere: keep the global accesses 16 bytes wide and realign through LDS
-            const uint64_t n_tiles = (outer * seg + kTileBytes - 1) / kTileBytes;
-            if (kl == FSTX_BATCH_MAX || tiles + n_tiles + kXcds > lim.launch) {
-                int rc = flush_lds();
-                if (rc < 0) return rc;
-            }
-            tl.job[kl] = LdsSliceJob{static_cast<char *>(d.dst), static_cast<const char *>(d.src),
-                                     pitch | ((uint64_t)ul << 56), (uint32_t)seg, (uint32_t)outer};
-            tiles_of[kl] = (n_tiles + kXcds - 1) / kXcds * kXcds; // whole eighths
-            tiles += tiles_of[kl];
-            if (seg < min_seg) min_seg = seg;
-            ++kl;
+        const fstx_join_src one{d.src, seg, pitch};
+        if ((mode == 2 || (mode == 1 && ul < 4)) && GatherBatch::takes(0, outer, &one, 1)) {
+            int rc = gather.add(d.dst, 0, outer, &one, 1);
+            if (rc < 0) return rc;
             continue;
         }
         const uint64_t seg_units = seg >> ul;
@@ -884,7 +779,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     }
     int rc = flush();
     if (rc < 0) return rc;
-    if ((rc = flush_lds()) < 0) return rc;
+    if ((rc = gather.flush()) < 0) return rc;
     return n_spans ? fstx_realign_copy_batch(spans, n_spans, stream) : 0;
 }
 
@@ -917,14 +812,22 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
     fstx_slice_desc dense[FSTX_BATCH_MAX];
     uint32_t n_dense = 0;
     const Limits lim = limits();
+    const int mode = fstx_internal::gather_mode();
+    GatherBatch gather(stream);
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_slice2d_desc &d = descs[i];
         if (d.outer == 0 || d.seg_bytes == 0) continue;
         if (!d.dst || !d.src) return -FSTX_E_INVAL;
         if (d.outer > 1 && (d.src_pitch < d.seg_bytes || d.dst_pitch < d.seg_bytes)) return -FSTX_E_INVAL;
         if (d.outer == 1 || d.dst_pitch == d.seg_bytes) {
-            // a dense destination: the plain slice extract (and its LDS and span forms) serves it
+            // a dense destination: the plain slice extract (and its span form) serves it
             dense[n_dense++] = fstx_slice_desc{d.dst, d.src, d.outer, d.seg_bytes, d.src_pitch};
+            continue;
+        }
+        const fstx_join_src one{d.src, d.seg_bytes, d.src_pitch};
+        if (mode != 0 && GatherBatch::takes(d.dst_pitch, d.outer, &one, 1)) {
+            int rc = gather.add(d.dst, d.dst_pitch, d.outer, &one, 1);
+            if (rc < 0) return rc;
             continue;
         }
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
@@ -949,6 +852,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
     }
     int rc = flush();
     if (rc < 0) return rc;
+    if ((rc = gather.flush()) < 0) return rc;
     return n_dense ? fstx_slice_copy_batch(dense, n_dense, stream) : 0;
 }
 
@@ -957,68 +861,32 @@ extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, cons
     if (n == 0 || rows == 0) return 0;
     if (!dst || !srcs) return -FSTX_E_INVAL;
     if (n > FSTX_JOIN_MAX) return -FSTX_E_TOO_MANY;
-    JoinTable t{};
-    t.dst = static_cast<char *>(dst);
-    uint64_t bits = (uint64_t)(uintptr_t)dst | 16u, row_bytes = 0, min_seg = ~0ull;
+    uint64_t row_bytes = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_join_src &s = srcs[i];
         if (s.seg_bytes == 0) continue;
         if (!s.src || (rows > 1 && s.src_pitch < s.seg_bytes) || s.seg_bytes >> 32) return -FSTX_E_INVAL;
-        bits |= (uint64_t)(uintptr_t)s.src | s.seg_bytes | s.src_pitch;
         row_bytes += s.seg_bytes;
-        if (s.seg_bytes < min_seg) min_seg = s.seg_bytes;
     }
     if (row_bytes == 0) return 0;
     if (dst_pitch == 0) dst_pitch = row_bytes;
     if (dst_pitch < row_bytes) return -FSTX_E_INVAL;
-    if (row_bytes >> 32 || rows >> 32) return -FSTX_E_RANGE;
-    const uint32_t ul = common_unit_log2(bits | dst_pitch);
-    t.dst_pitch = dst_pitch;
-    t.rows = (uint32_t)rows;
-    t.unit_log2 = ul;
-    // rows per chunk: the shortest block still fills sixteen wavefronts, so that the idle
-    // lanes at the end of each source's share of a chunk stay below a few percent
-    uint64_t rpc = (16ull * kBlock + (min_seg >> ul) - 1) / (min_seg >> ul);
-    if (rpc > rows) rpc = rows;
-    const Limits lim = limits();
-    auto waves_of = [&](uint64_t rows_per_chunk) {
-        uint64_t w = 0;
-        for (uint32_t i = 0; i < n; ++i)
-            w += (rows_per_chunk * (srcs[i].seg_bytes >> ul) + kBlock - 1) / kBlock;
-        return w;
-    };
-    // ... unless a very short block next to very long ones would make one chunk larger than a launch
-    while (rpc > 1 && (waves_of(rpc) > lim.launch || rpc * (row_bytes >> ul) > lim.units())) rpc /= 2;
-    t.rows_per_chunk = (uint32_t)rpc;
-    uint64_t waves = 0, col = 0;
+    if (fstx_internal::gather_mode() != 0 && GatherBatch::takes(dst_pitch, rows, srcs, n)) {
+        GatherBatch gather(stream);
+        int rc = gather.add(dst, dst_pitch, rows, srcs, n);
+        return rc < 0 ? rc : gather.flush();
+    }
+    // some block is narrower than 16 bytes: every block on its own into its columns of the joined rows
+    fstx_slice2d_desc each[FSTX_JOIN_MAX];
+    uint32_t m = 0;
+    uint64_t col = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const fstx_join_src &s = srcs[i];
         if (s.seg_bytes == 0) continue;
-        const uint64_t units = rpc * (s.seg_bytes >> ul);
-        if (units > lim.units()) return -FSTX_E_RANGE;
-        t.wave_begin[t.n] = (uint32_t)waves;
-        t.src[t.n] = JoinSrc{static_cast<const char *>(s.src), s.src_pitch, (uint32_t)(s.seg_bytes >> ul), (uint32_t)col, 0};
-        waves += (units + kBlock - 1) / kBlock;
+        each[m++] = fstx_slice2d_desc{static_cast<char *>(dst) + col, s.src, rows, s.seg_bytes, s.src_pitch, dst_pitch};
         col += s.seg_bytes;
-        ++t.n;
     }
-    if (waves == 0 || waves > lim.launch) return -FSTX_E_RANGE; // one joined row is more than a launch holds
-    t.waves_per_chunk = (uint32_t)waves;
-    // as many chunks per launch as the grid allows; the next launch continues further down
-    const uint64_t chunks_per_launch = lim.launch / waves;
-    for (uint64_t row = 0; row < rows; row += chunks_per_launch * rpc) {
-        const uint64_t part = rows - row < chunks_per_launch * rpc ? rows - row : chunks_per_launch * rpc;
-        JoinTable tt = t;
-        tt.dst += row * dst_pitch;
-        tt.rows = (uint32_t)part;
-        for (uint32_t j = 0; j < tt.n; ++j) tt.src[j].src += row * tt.src[j].src_pitch;
-        const uint64_t grid = (part + rpc - 1) / rpc * waves;
-        if (!grid_fits(grid)) return -FSTX_E_RANGE;
-        hipLaunchKernelGGL(join_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream), tt);
-        int rc = fstx_internal::check_launch("join_kernel");
-        if (rc < 0) return rc;
-    }
-    return 0;
+    return fstx_slice_copy2d_batch(each, m, stream);
 }
 
 extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {

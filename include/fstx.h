@@ -5,7 +5,7 @@
  * One shared library (libfstx.so, HIP, gfx950) holds
  *   - the file -> pinned ring -> HBM copy pipeline, and
  *   - the kernels that post-process tensors in HBM (realign copy, slice
- *     extract in its dense, strided-destination and LDS-staged forms, down-cast).
+ *     extract into dense, pitched and joined destinations, down-cast).
  * Every entry point takes plain pointers and sizes; there are no C++ or torch
  * types in the signatures, so the library binds from ctypes, cgo, JNI or any
  * other FFI.  Each declaration names the interface of the reference
@@ -20,6 +20,10 @@
  *     stream.  Kernel entry points only enqueue work; they do not synchronize.
  *   - Device pointers must belong to the device that is current on the
  *     calling thread (kernels) or to the context's device (reads).
+ *   - A strided source (`outer` segments `src_pitch` apart) must be readable from the
+ *     first byte of its first segment to the last byte of its last one, bytes between the
+ *     segments included: it is a block of a tensor.  The kernels never touch a byte before
+ *     or behind that range, and never write a destination byte that is not a segment's.
  */
 #ifndef FSTX_H
 #define FSTX_H
@@ -217,8 +221,10 @@ int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, void *strea
  * rank's shard of a row-major tensor cut along a dimension: for shape
  * [.., S, ..] cut at dim d into blocks of bs, outer = prod(shape[:d]),
  * src_pitch = S * inner_bytes, seg_bytes = rows_of_this_rank * inner_bytes and
- * src already points at the rank's first row.  Replaces the per-rank
- * t[slices].contiguous() of LazyTensorFactory.shuffle (tensor_factory.py:168-175). */
+ * src already points at the rank's first row.  Nothing has to be aligned: segments
+ * of 16 bytes and more move as 16-byte vectors whatever the addresses, lengths and
+ * pitches are.  Replaces the per-rank t[slices].contiguous() of
+ * LazyTensorFactory.shuffle (tensor_factory.py:168-175). */
 int fstx_slice_copy(void *dst, const void *src, uint64_t outer, uint64_t seg_bytes,
                     uint64_t src_pitch, void *stream);
 
@@ -263,8 +269,9 @@ typedef struct fstx_join_src {
 /* Fused slice + concatenate along an inner dimension: row r of the destination (rows
  * dst_pitch bytes apart; 0 = dense, sum(seg_bytes)) is the r-th segments of the n sources
  * side by side.  Same result as n descriptors of fstx_slice_copy2d_batch, but the
- * workgroups sweep the destination in row order (a few rows of all sources at a time), so
- * its writes stay sequential (measured 5 to 7 % faster than the strided form).
+ * destination is written front to back in whole 16-byte vectors -- a vector that holds the
+ * end of one block and the beginning of the next is put together in registers -- whatever
+ * the widths and alignments of the blocks are.
  * Replaces the contiguous() + torch.cat of LazyTensorFactory.shuffle_multi_cols
  * (tensor_factory.py:194-259).  n <= FSTX_JOIN_MAX. */
 int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,

@@ -202,5 +202,5 @@ int copy_to_device_async(void *dev_dst, const void *host_src, size_t bytes, stre
 
 namespace fstx_internal {
 int check_launch(const char *) { return 0; }
-bool lds_path_disabled() { return false; }
+int gather_mode() { return 1; }
 } // namespace fstx_internal

@@ -1,0 +1,111 @@
+// SPDX-License-Identifier: Apache-2.0
+//
+// TEST INFRASTRUCTURE.  Runs the gather kernel's lane logic (fstx_gather_core.h, the same
+// source the GPU kernel is built from) lane by lane on the CPU over caller-provided buffers,
+// with every memory access checked: a load must lie inside one source's block (first byte of
+// its first segment to last byte of its last), a store must hit payload bytes of the destination, and every payload byte must be
+// written exactly once.  Lets the index arithmetic be swept over odd shapes and alignments
+// without a GPU.  Not part of the shipped library.
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "fstx_gather_core.h"
+
+using namespace fstx_gather;
+
+namespace {
+
+struct SimMem {
+    const Job *job;
+    const Src *srcs;
+    std::vector<uint8_t> *written; // per destination position: times written
+    char *dst_lo;                  // allocation bounds of the destination
+    char *dst_hi;
+    int64_t errors = 0;
+
+    Vec16 load16_stream(const char *p) { return load16(p); }
+    // a load must lie inside one source's block: from the first byte of its first segment to the
+    // last byte of its last segment (what the caller guarantees to be readable)
+    Vec16 load16(const char *p) {
+        bool ok = false;
+        for (uint32_t k = 0; k < job->nsrc && !ok; ++k) {
+            const Src &s = srcs[k];
+            ok = p >= s.src && p + kVec <= s.src + (uint64_t)(job->rows - 1) * s.pitch + s.seg;
+        }
+        Vec16 v = {{0, 0, 0, 0}};
+        if (!ok) {
+            ++errors;
+            return v;
+        }
+        std::memcpy(&v, p, kVec);
+        return v;
+    }
+    void note(char *p) {
+        if (p < job->dst || p >= dst_hi) {
+            ++errors;
+            return;
+        }
+        const uint64_t pos = (uint64_t)(p - job->dst);
+        const uint64_t row = pos / job->dst_pitch, c = pos % job->dst_pitch;
+        if (row >= job->rows || c >= job->row_bytes || (*written)[pos] == 255) {
+            ++errors;
+            return;
+        }
+        ++(*written)[pos];
+    }
+    void store16(char *p, Vec16 v) {
+        if (((uintptr_t)p & 15) || p < dst_lo || p + kVec > dst_hi) {
+            ++errors;
+            return;
+        }
+        for (uint32_t i = 0; i < kVec; ++i) note(p + i);
+        std::memcpy(p, &v, kVec);
+    }
+    void store8(char *p, unsigned char b) {
+        note(p);
+        if (p >= dst_lo && p < dst_hi) *p = (char)b;
+    }
+};
+
+} // namespace
+
+// Runs one job: `n` sources (src[i], seg[i], pitch[i]) into dst rows `dst_pitch` apart.
+// Returns 0 when every access was legal and every payload byte was written exactly once,
+// -1 when the shape is outside the kernel's domain, else the number of violations.
+extern "C" int64_t fstx_gather_sim(char *dst, uint64_t dst_capacity_before, uint64_t dst_capacity_after, uint64_t dst_pitch,
+                                   uint64_t rows, const char *const *src, const uint64_t *seg, const uint64_t *pitch,
+                                   uint32_t n, int general) {
+    std::vector<Src> srcs(n);
+    uint64_t col = 0, min_seg = ~0ull, equal = n ? seg[0] : 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        srcs[i] = Src{src[i], pitch[i], (uint32_t)seg[i], (uint32_t)col, 0};
+        col += seg[i];
+        if (seg[i] < min_seg) min_seg = seg[i];
+        if (seg[i] != equal) equal = 0;
+    }
+    if (dst_pitch == 0) dst_pitch = col;
+    if (!shape_ok(dst_pitch, col, min_seg) || rows == 0 || rows > rows_per_job(dst_pitch, col)) return -1;
+    // the kernel's table holds sources 1 .. n-1; source 0 travels in the job
+    const uint32_t more0 = 3; // somewhere inside a larger table
+    std::vector<Src> more(more0 + n);
+    for (uint32_t i = 1; i < n; ++i) more[more0 + i - 1] = srcs[i];
+    const Job jb = make_job(dst, dst_pitch, col, rows, srcs[0], more0, n, n > 1 ? equal : 0);
+    std::vector<uint8_t> written((rows - 1) * dst_pitch + col, 0);
+    SimMem mem{&jb, srcs.data(), &written, dst - dst_capacity_before, dst + dst_capacity_after};
+    const uint64_t tiles = tiles_of(jb);
+    // the leanest variant the job allows, as the library picks it (general = 1 forces the full one)
+    const bool multi = n > 1 || general, pitched = dst_pitch != col || general;
+    for (uint64_t t = 0; t < tiles; ++t)
+        for (uint32_t lane = 0; lane < kLanes; ++lane) {
+            if (multi && pitched) gather_lane<true, true>(jb, more.data(), (uint32_t)t, lane, mem);
+            else if (multi) gather_lane<true, false>(jb, more.data(), (uint32_t)t, lane, mem);
+            else if (pitched) gather_lane<false, true>(jb, more.data(), (uint32_t)t, lane, mem);
+            else gather_lane<false, false>(jb, more.data(), (uint32_t)t, lane, mem);
+        }
+    int64_t bad = mem.errors;
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t c = 0; c < col; ++c)
+            if (written[r * dst_pitch + c] != 1) ++bad;
+    return bad;
+}

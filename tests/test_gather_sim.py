@@ -1,0 +1,132 @@
+# SPDX-License-Identifier: Apache-2.0
+"""The gather kernel's lane logic on the CPU, every access checked.
+
+``tests/kernel_sim`` compiles ``csrc/fstx_gather_core.h`` -- the source the GPU kernel is
+built from -- for the host and runs it lane by lane: a load must lie inside one segment of
+one source, a store inside the destination's payload, every payload byte must be written
+exactly once, and the result must equal numpy's own gather of the same bytes (the oracle's
+``shard_bytes`` rule: ``outer`` segments of ``seg`` bytes read ``pitch`` apart).  Sweeps odd
+segment lengths, pitches, source and destination alignments, joins of unequal blocks and
+pitched destinations -- the shapes that cannot be tried blindly on a GPU.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SIM_DIR = os.path.join(HERE, "kernel_sim")
+
+
+@pytest.fixture(scope="module")
+def sim():
+    so = os.path.join(SIM_DIR, "libfstx_kernel_sim.so")
+    src = [os.path.join(SIM_DIR, "gather_sim.cpp"), os.path.join(HERE, "..", "fastsafetensors_amd", "csrc", "fstx_gather_core.h")]
+    if not os.path.exists(so) or any(os.path.getmtime(s) > os.path.getmtime(so) for s in src):
+        subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
+    lib = ctypes.CDLL(so)
+    lib.fstx_gather_sim.restype = ctypes.c_int64
+    lib.fstx_gather_sim.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64,
+                                    ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_uint64),
+                                    ctypes.POINTER(ctypes.c_uint64), ctypes.c_uint32, ctypes.c_int]
+    return lib
+
+
+def run_case(sim, rng, rows, segs, pitches, src_mis, dst_mis, gap):
+    """One job; returns (violations, result equals numpy's gather)."""
+    n = len(segs)
+    srcs, views = [], []
+    for seg, pitch, mis in zip(segs, pitches, src_mis):
+        raw = rng.integers(0, 256, rows * pitch + 64, dtype=np.uint8)
+        off = (-raw.ctypes.data) % 16 + mis  # the block's first byte sits `mis` past a 16-byte boundary
+        srcs.append(raw)
+        views.append((raw.ctypes.data + off, off))
+    row_bytes = sum(segs)
+    dst_pitch = row_bytes + gap
+    span = (rows - 1) * dst_pitch + row_bytes
+    guard = 64
+    buf = np.full(span + 2 * guard + 32, 0xA5, dtype=np.uint8)
+    d_off = guard + (-(buf.ctypes.data + guard)) % 16 + dst_mis
+    ptrs = (ctypes.c_void_p * n)(*[v[0] for v in views])
+    seg_a = (ctypes.c_uint64 * n)(*segs)
+    pitch_a = (ctypes.c_uint64 * n)(*pitches)
+    # the variant the library would pick for the job, and the fully general one: same bytes either way
+    general = sim.fstx_gather_sim(buf.ctypes.data + d_off, d_off, buf.size - d_off, dst_pitch if gap else 0, rows, ptrs,
+                                  seg_a, pitch_a, n, 1)
+    first = buf.copy()
+    buf[:] = 0xA5
+    bad = sim.fstx_gather_sim(buf.ctypes.data + d_off, d_off, buf.size - d_off, dst_pitch if gap else 0, rows, ptrs, seg_a,
+                              pitch_a, n, 0)
+    if general != bad or not np.array_equal(first, buf):
+        bad = bad if bad else 999
+    want = np.full_like(buf, 0xA5)
+    for r in range(rows):
+        col = 0
+        for (addr, off), raw, seg, pitch in zip(views, srcs, segs, pitches):
+            want[d_off + r * dst_pitch + col : d_off + r * dst_pitch + col + seg] = raw[off + r * pitch : off + r * pitch + seg]
+            col += seg
+    return bad, np.array_equal(buf, want)
+
+
+@pytest.mark.parametrize("seg,pitch", [(16, 16 + 1), (17, 40), (31, 31 + 33), (64, 100), (70, 282), (254, 1018), (1022, 4090),
+                                       (1024, 4096), (1040, 2081), (2046, 8180), (2048, 8190), (4094, 16376), (6912, 27648)])
+def test_one_source_every_alignment(sim, seg, pitch):
+    """A rank's block of one tensor: all 16 x 16 combinations of source and destination alignment."""
+    rng = np.random.default_rng(seg * 7 + pitch)
+    rows = max(3, min(40, 9000 // seg + 2))
+    for src_mis in range(16):
+        for dst_mis in range(16):
+            bad, same = run_case(sim, rng, rows, [seg], [pitch], [src_mis], dst_mis, 0)
+            assert bad == 0 and same, (seg, pitch, src_mis, dst_mis, bad)
+
+
+def test_joins_of_unequal_and_equal_blocks(sim):
+    rng = np.random.default_rng(11)
+    cases = [
+        ([1022, 254, 254], [4090, 1018, 1018]),          # q, k, v blocks of odd widths
+        ([2046] * 4, [8190] * 4),                        # fp8 [N, 8190] cut in 4, last rank
+        ([6912] * 14, [27648] * 14),                     # 14 down_proj column blocks (16-byte multiples)
+        ([16, 17, 16, 33], [100, 50, 16, 99]),           # shortest legal segments, one source dense (pitch == seg)
+        ([70, 70, 70], [282, 282, 282]),
+        ([1500, 20, 1500], [1500, 4096, 3001]),
+        ([24] * 24, [24 * 5] * 24),                      # the most sources one call takes
+    ]
+    for segs, pitches in cases:
+        for trial in range(6):
+            mis = [int(x) for x in rng.integers(0, 16, len(segs))]
+            bad, same = run_case(sim, rng, int(rng.integers(1, 30)), segs, pitches, mis, int(rng.integers(0, 16)), 0)
+            assert bad == 0 and same, (segs, pitches, mis, bad)
+
+
+def test_pitched_destinations(sim):
+    """Rows of the destination further apart than their payload: the gap is never written,
+    whatever its size (smaller than a vector, a vector, several)."""
+    rng = np.random.default_rng(12)
+    for segs, pitches in [([2046], [8180]), ([100, 28], [300, 28]), ([6912] * 3, [27648] * 3), ([16], [16]), ([40, 1000], [77, 1003])]:
+        for gap in (1, 2, 7, 15, 16, 17, 31, 32, 100, 1024, 5000):
+            mis = [int(x) for x in rng.integers(0, 16, len(segs))]
+            bad, same = run_case(sim, rng, int(rng.integers(1, 12)), segs, pitches, mis, int(rng.integers(0, 16)), gap)
+            assert bad == 0 and same, (segs, gap, bad)
+
+
+def test_random_geometries(sim):
+    rng = np.random.default_rng(13)
+    for trial in range(400):
+        n = int(rng.choice([1, 1, 1, 2, 3, 5]))
+        segs = [int(rng.integers(16, 3000)) for _ in range(n)]
+        if rng.random() < 0.3:
+            segs = [segs[0]] * n
+        pitches = [s + int(rng.integers(0, 2000)) for s in segs]
+        rows = int(rng.integers(1, max(2, 20000 // sum(segs))))
+        gap = int(rng.choice([0, 0, 0, int(rng.integers(1, 300))]))
+        mis = [int(x) for x in rng.integers(0, 16, n)]
+        bad, same = run_case(sim, rng, rows, segs, pitches, mis, int(rng.integers(0, 16)), gap)
+        assert bad == 0 and same, (trial, segs, pitches, rows, gap, mis, bad)
+
+
+def test_shapes_outside_the_kernels_domain_are_refused(sim):
+    rng = np.random.default_rng(14)
+    assert run_case(sim, rng, 4, [15], [100], [0], 0, 0)[0] == -1      # a segment shorter than a vector
+    assert run_case(sim, rng, 4, [64, 8], [64, 8], [0, 0], 0, 0)[0] == -1

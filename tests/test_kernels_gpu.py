@@ -190,10 +190,11 @@ def test_slice_batch_and_round_trip_full_size_c4(dev):
             assert torch.equal(parts[rank].view(torch.int16), t[sl].contiguous().view(torch.int16))
 
 
-def test_slice_odd_shapes_go_through_lds(dev):
+def test_slice_odd_shapes(dev):
     """Segments that are not multiples of 16 bytes (odd column counts, 1-byte dtypes,
-    shifted sources): the LDS-staged kernel, against torch's own slicing on the GPU,
-    and against the direct small-unit kernel (FSTX_NO_LDS_SLICE=1)."""
+    shifted sources, destinations at odd addresses): the gather kernel, against torch's own
+    slicing on the GPU, and against the small-unit kernels (FSTX_GATHER_MODE=0) and the
+    gather kernel forced onto every shape (FSTX_GATHER_MODE=2)."""
     import os
 
     rng = np.random.default_rng(11)
@@ -213,24 +214,27 @@ def test_slice_odd_shapes_go_through_lds(dev):
                 inner = int(np.prod(shape[dim + 1 :], dtype=np.int64)) * item
                 outer = int(np.prod(shape[:dim], dtype=np.int64))
                 outs = []
-                for no_lds in ("0", "1"):
-                    os.environ["FSTX_NO_LDS_SLICE"] = no_lds
-                    got = torch.full((want.numel() + 32,), 77, dtype=dtype, device=dev)
-                    _native.slice_copy(got.data_ptr() + 16 * item * 0 + 0, t.data_ptr() + lo * inner, outer,
-                                       (hi_ - lo) * inner, shape[dim] * inner, stream())
-                    outs.append(got)
-                os.environ.pop("FSTX_NO_LDS_SLICE")
-                for got in outs:
-                    assert torch.equal(got[: want.numel()].view(want.shape), want), (shape, dtype, rank, shift)
-                    assert (got[want.numel() :] == 77).all(), "wrote past the end of the shard"
+                for mode in ("1", "0", "2"):
+                    os.environ["FSTX_GATHER_MODE"] = mode
+                    for lead in (0, 1, 5):  # the destination's first element: aligned, and off by 1 and 5 elements
+                        got = torch.full((want.numel() + 32,), 77, dtype=dtype, device=dev)
+                        _native.slice_copy(got.data_ptr() + lead * item, t.data_ptr() + lo * inner, outer,
+                                           (hi_ - lo) * inner, shape[dim] * inner, stream())
+                        outs.append((got, lead))
+                os.environ.pop("FSTX_GATHER_MODE")
+                for got, lead in outs:
+                    assert torch.equal(got[lead : lead + want.numel()].view(want.shape), want), (shape, dtype, rank, shift, lead)
+                    assert (got[:lead] == 77).all() and (got[lead + want.numel() :] == 77).all(), "wrote outside the shard"
 
 
-def test_slice_lds_random_geometry_in_one_batch(dev):
-    """Byte-level sweep of the LDS-staged kernel: segment lengths around the tile size and
-    its fractions, odd pitches, every source alignment, jobs of very different segment
-    lengths sharing one launch (the launch's LDS size follows the shortest segment)."""
+def test_gather_random_geometry_in_one_batch(dev):
+    """Byte-level sweep of the gather kernel: segment lengths from the shortest it takes (16
+    bytes; 9 and 15 go to the small-unit kernel) over the tile size and its fractions, odd
+    pitches, every source and destination alignment, jobs of very different segment lengths
+    sharing one launch."""
     rng = np.random.default_rng(23)
-    segs = [64, 65, 79, 81, 127, 129, 255, 511, 513, 1023, 1025, 2046, 2047, 2049, 2050, 4094, 4095, 4097, 6001, 8191]
+    segs = [9, 15, 16, 17, 31, 33, 64, 65, 79, 81, 127, 129, 255, 511, 513, 1023, 1025, 2046, 2047, 2049, 2050, 4094, 4095,
+            4097, 6001, 8191]
     for _ in range(6):
         jobs, checks = [], []
         for _j in range(24):
@@ -238,15 +242,17 @@ def test_slice_lds_random_geometry_in_one_batch(dev):
             pitch = seg + int(rng.choice([1, 2, 3, 7, 13, 16, 17, 100, 1001]))
             outer = int(rng.integers(2, 40)) if seg < 3000 else int(rng.integers(2, 6))
             shift = int(rng.integers(0, 16))
-            src = torch.randint(0, 255, (shift + outer * pitch + 32,), dtype=torch.uint8, device=dev)
-            dst = torch.full((outer * seg + 48,), 201, dtype=torch.uint8, device=dev)
-            jobs.append((dst.data_ptr(), src.data_ptr() + shift, outer, seg, pitch))
-            checks.append((src, dst, shift, outer, seg, pitch))
+            lead = int(rng.integers(0, 16))
+            # the source tensor ends with its last segment: a load that strayed past it would leave the allocation's payload
+            src = torch.randint(0, 255, (shift + (outer - 1) * pitch + seg,), dtype=torch.uint8, device=dev)
+            dst = torch.full((lead + outer * seg + 48,), 201, dtype=torch.uint8, device=dev)
+            jobs.append((dst.data_ptr() + lead, src.data_ptr() + shift, outer, seg, pitch))
+            checks.append((src, dst, shift, lead, outer, seg, pitch))
         _native.slice_copy_batch(jobs, stream())
-        for src, dst, shift, outer, seg, pitch in checks:
-            want = src[shift : shift + outer * pitch].view(outer, pitch)[:, :seg].reshape(-1)
-            assert torch.equal(dst[: outer * seg], want), (seg, pitch, outer, shift)
-            assert (dst[outer * seg :] == 201).all(), "wrote past the end"
+        for src, dst, shift, lead, outer, seg, pitch in checks:
+            want = torch.stack([src[shift + r * pitch : shift + r * pitch + seg] for r in range(outer)]).reshape(-1)
+            assert torch.equal(dst[lead : lead + outer * seg], want), (seg, pitch, outer, shift, lead)
+            assert (dst[:lead] == 201).all() and (dst[lead + outer * seg :] == 201).all(), "wrote outside the block"
 
 
 def test_slice2d_strided_destination(dev):
@@ -344,7 +350,7 @@ def test_tensors_beyond_4_gib(dev):
     _native.slice_copy(rowcut.data_ptr(), t.data_ptr() + block * cols * 2, 1, block * cols * 2, rows * cols * 2, stream())
     assert torch.equal(rowcut, t[block:])
     del rowcut, t
-    # an odd column count: the LDS-staged kernel with more than 4 GiB per job (64-bit tile arithmetic)
+    # an odd column count: the gather kernel with more than 4 GiB per tensor (cut into jobs of 32-bit positions)
     rows, cols = 80000, 65537
     t = torch.randint(-30000, 30000, (rows, cols), dtype=torch.int16, device=dev)
     block = -(-cols // 2)
@@ -363,11 +369,11 @@ def test_tensors_beyond_4_gib(dev):
     rows, cols = 80000, 65537
     t = torch.randint(0, 255, (rows, cols), dtype=torch.uint8, device=dev)
     cut = torch.empty((rows, cols - 1), dtype=torch.uint8, device=dev)
-    os.environ["FSTX_NO_LDS_SLICE"] = "1"
+    os.environ["FSTX_GATHER_MODE"] = "0"
     try:
         _native.slice_copy(cut.data_ptr(), t.data_ptr(), rows, cols - 1, cols, stream())
     finally:
-        os.environ.pop("FSTX_NO_LDS_SLICE")
+        os.environ.pop("FSTX_GATHER_MODE")
     assert torch.equal(cut, t[:, :-1])
     cut.zero_()
     wide = torch.zeros((rows, cols + 2), dtype=torch.uint8, device=dev)
@@ -396,8 +402,8 @@ def test_cutting_into_jobs_and_launches(dev, monkeypatch):
     through the code that cuts spans, tensors and joins into several jobs and launches."""
     monkeypatch.setenv("FSTX_MAX_BLOCKS_PER_LAUNCH", "4096")
     test_realign_batch_many_jobs(dev)
-    test_slice_odd_shapes_go_through_lds(dev)
-    test_slice_lds_random_geometry_in_one_batch(dev)
+    test_slice_odd_shapes(dev)
+    test_gather_random_geometry_in_one_batch(dev)
     test_slice2d_strided_destination(dev)
     test_join_copy_matches_cat(dev)
     # one span, one strided tensor, one join and one conversion that are each many launches long
