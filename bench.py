@@ -19,7 +19,8 @@ Next to it, on the same line:
                   tensors (config C4, TP=4, all four ranks in turn), timed with
                   events on the stream the launches go to; ``kernels`` carries the
                   other kernels as well (realign on config C2's data section, row
-                  cuts, joined column cuts, odd shapes through LDS, fp32 -> bf16).
+                  cuts, joined column cuts, odd shapes and odd joins through the gather
+                  kernel, fp32 -> bf16).
 ``tp_extract``, ``multi_cols``, ``iterate_weights``, ``downcast_on_load``
                   the callers around the path, timed through the Python API.
 ``pipeline``      measured ceilings of this box -- O_DIRECT read rate of the same
@@ -561,7 +562,7 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
             raise SystemExit("bench: joined column blocks differ from slicing + cat")
     out["slice_join_columns"] = {
         "workload": f"C4 down_proj [{rows}, {cols}] column blocks of {len(downs)} layers cut into one joined [{rows}, {blk * len(downs)}] "
-                    f"tensor per rank (one launch of join_kernel per rank)",
+                    f"tensor per rank (one launch of gather_kernel per rank)",
         "launches_timed": len(jt), "avg_launch_ms": sum(jt) / len(jt), "bytes_per_launch": jb,
         "achieved_GBps": jb / 1e6 / (sum(jt) / len(jt)),
     }
@@ -575,33 +576,66 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
     del srcs, keep, launches
     torch.cuda.empty_cache()
 
-    # -- slice extract on shapes whose rows are not multiples of 16 bytes: the LDS-staged
-    #    kernel against the direct kernel at the small unit such shapes force
+    # -- slice extract on shapes whose rows are not multiples of 16 bytes: the gather kernel
+    #    (16-byte loads at the data's own byte address), and, for the record, the small-unit
+    #    kernels such shapes were left to before it existed (FSTX_GATHER_MODE=0)
     odd = {}
     # (inputs of 0.5 GB each: larger than the 256 MB memory-side cache, so that repeated launches
     #  are served by HBM)
-    for label, shape, tdt in [("bf16 [65536, 4090] cut in 4 along dim 1 (2046-byte segments, 8180-byte pitch)", (65536, 4090), torch.int16),
-                              ("fp8 [65536, 8190] cut in 4 along dim 1 (2048-byte segments, 8190-byte pitch)", (65536, 8190), torch.uint8),
-                              ("bf16 [32768, 8188] cut in 4 along dim 1 (4094-byte segments, 16376-byte pitch)", (32768, 8188), torch.int16)]:
+    for label, shape, tdt, lead in [
+            ("bf16 [65536, 4090] cut in 4 along dim 1 (2046-byte segments, 8180-byte pitch)", (65536, 4090), torch.int16, 0),
+            ("fp8 [65536, 8190] cut in 4 along dim 1 (2048-byte segments, 8190-byte pitch)", (65536, 8190), torch.uint8, 0),
+            ("bf16 [32768, 8188] cut in 4 along dim 1 (4094-byte segments, 16376-byte pitch)", (32768, 8188), torch.int16, 0),
+            ("bf16 [32768, 8188] cut in 4 along dim 1 into destinations 6 bytes off a 16-byte boundary", (32768, 8188), torch.int16, 3)]:
         t = torch.randint(0, 100, shape, dtype=tdt, device=dev)
         item = t.element_size()
         block = -(-shape[1] // world)
-        dsts = [torch.empty((shape[0], min(block, shape[1] - r * block)), dtype=tdt, device=dev) for r in range(world)]
-        jobs = [(dsts[r].data_ptr(), t.data_ptr() + r * block * item, shape[0], dsts[r].shape[1] * item, shape[1] * item)
+        widths = [min(block, shape[1] - r * block) for r in range(world)]
+        flats = [torch.empty(shape[0] * w + 64, dtype=tdt, device=dev) for w in widths]
+        dsts = [f[lead : lead + shape[0] * w].view(shape[0], w) for f, w in zip(flats, widths)]
+        jobs = [(dsts[r].data_ptr(), t.data_ptr() + r * block * item, shape[0], widths[r] * item, shape[1] * item)
                 for r in range(world)]
         nb = 2 * sum(d.numel() * item for d in dsts)
         res = {}
-        for mode, env in (("lds_staged", "0"), ("direct_small_unit", "1")):
-            os.environ["FSTX_NO_LDS_SLICE"] = env
+        for mode, env in (("gather_kernel", "1"), ("small_unit_kernels", "0")):
+            os.environ["FSTX_GATHER_MODE"] = env
             _native.slice_copy_batch(jobs, stream)
             ms = timed([lambda: _native.slice_copy_batch(jobs, stream)] * 5)
             res[mode] = {"avg_launch_ms": sum(ms) / len(ms), "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
             if not all(torch.equal(dsts[r], t[:, r * block : (r + 1) * block]) for r in range(world)):
                 raise SystemExit(f"bench: odd-shape slice ({mode}) differs from torch's slice")
-        os.environ.pop("FSTX_NO_LDS_SLICE")
+        os.environ.pop("FSTX_GATHER_MODE")
         odd[label] = dict(res, bytes_per_launch=nb)
-        del t, dsts
+        del t, dsts, flats
     out["slice_extract_odd_shapes"] = odd
+
+    # -- get_multi_cols along dim 1 on odd widths: the rank's column blocks of several tensors cut
+    #    straight into one joined tensor (one launch per rank; a destination vector that holds the end
+    #    of one block and the start of the next is put together in registers)
+    odd_joins = {}
+    for label, shape, tdt, count in [("6 x fp8 [32768, 8190], column blocks of a rank joined along dim 1", (32768, 8190), torch.uint8, 6),
+                                     ("8 x bf16 [16384, 4090], column blocks of a rank joined along dim 1", (16384, 4090), torch.int16, 8)]:
+        ts = [torch.randint(0, 100, shape, dtype=tdt, device=dev) for _ in range(count)]
+        item = ts[0].element_size()
+        block = -(-shape[1] // world)
+        widths = [min(block, shape[1] - r * block) for r in range(world)]
+        outs = [torch.empty((shape[0], count * w), dtype=tdt, device=dev) for w in widths]
+        jsrc = [[(t.data_ptr() + r * block * item, widths[r] * item, shape[1] * item) for t in ts] for r in range(world)]
+        nb = 2 * sum(o.numel() * item for o in outs) / world
+        res = {}
+        for mode, env in (("gather_kernel", "1"), ("small_unit_kernels", "0")):
+            os.environ["FSTX_GATHER_MODE"] = env
+            for r in range(world):
+                _native.join_copy(outs[r].data_ptr(), shape[0], jsrc[r], stream)
+            ms = timed([lambda r=r: _native.join_copy(outs[r].data_ptr(), shape[0], jsrc[r], stream) for r in range(world)] * 3)
+            res[mode] = {"avg_launch_ms": sum(ms) / len(ms), "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
+            for r in range(world):
+                if not torch.equal(outs[r], torch.cat([t[:, r * block : (r + 1) * block] for t in ts], dim=1)):
+                    raise SystemExit(f"bench: odd join ({mode}) differs from slicing + cat")
+        os.environ.pop("FSTX_GATHER_MODE")
+        odd_joins[label] = dict(res, bytes_per_launch=nb)
+        del ts, outs
+    out["join_odd_columns"] = odd_joins
 
     # -- realign: config C2's data section shifted by header_length % 16 = 10 bytes
     n = 709_646_336
