@@ -409,7 +409,7 @@ def bench_multi_cols(files: List[str], world: int, threads: int, block_kb: int) 
         p = f"model.layers.{i}."
         groups.append([p + f"self_attn.{x}_proj.weight" for x in "qkv"])
         groups.append([p + f"mlp.{x}_proj.weight" for x in ("gate", "up")])
-    secs, moved, checked = [], 0, 0
+    secs, secs_singly, moved, checked = [], [], 0, 0
     for rank in range(world):
         loader = SafeTensorsFileLoader(StubProcessGroup(rank, world), "cuda:0", max_threads=threads,
                                        block_size_kb=block_kb)
@@ -418,7 +418,13 @@ def bench_multi_cols(files: List[str], world: int, threads: int, block_kb: int) 
         bufs.auto_mem_delete = False
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        outs = [bufs.get_multi_cols(names, dim=0) for names in groups]
+        singly = [bufs.get_multi_cols(names, dim=0) for names in groups]  # one call, one launch per group
+        torch.cuda.synchronize()
+        secs_singly.append(time.perf_counter() - t0)
+        del singly
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = bufs.get_multi_cols_many(groups, dim=0)  # one call: a few launches per file
         torch.cuda.synchronize()
         secs.append(time.perf_counter() - t0)
         moved += sum(2 * t.get_raw().numel() * t.get_raw().element_size() for t in outs)
@@ -436,9 +442,11 @@ def bench_multi_cols(files: List[str], world: int, threads: int, block_kb: int) 
         loader.close()
     whole.close()
     whole_loader.close()
-    return {"workload": f"get_multi_cols of [q,k,v] and [gate,up] (dim 0) for {len(layers)} layers, each of {world} ranks",
-            "calls_per_rank": len(groups), "seconds_per_rank": secs, "algorithmic_bytes": moved,
-            "GBps": moved / 1e9 / sum(secs), "joined_tensors_compared": checked}
+    return {"workload": f"get_multi_cols_many of [q,k,v] and [gate,up] (dim 0) for {len(layers)} layers ({len(groups)} groups in one "
+                        f"call), each of {world} ranks",
+            "groups_per_rank": len(groups), "seconds_per_rank": secs, "algorithmic_bytes": moved,
+            "GBps": moved / 1e9 / sum(secs), "joined_tensors_compared": checked,
+            "one_call_per_group": {"seconds_per_rank": secs_singly, "GBps": moved / 1e9 / sum(secs_singly)}}
 
 
 def bench_iterate_weights(files: List[str], threads: int, verify) -> dict:

@@ -8,6 +8,7 @@ device-buffer handle, and a handful of free functions.  There is no Python or
 CPU substitute for anything in here: if the library is missing, loading raises.
 """
 
+import array
 import ctypes
 import os
 import threading
@@ -98,6 +99,17 @@ class FstxJoinSrc(ctypes.Structure):
     _fields_ = [("src", ctypes.c_void_p), ("seg_bytes", ctypes.c_uint64), ("src_pitch", ctypes.c_uint64)]
 
 
+class FstxJoinDesc(ctypes.Structure):
+    _fields_ = [
+        ("dst", ctypes.c_void_p),
+        ("dst_pitch", ctypes.c_uint64),
+        ("rows", ctypes.c_uint64),
+        ("srcs", ctypes.POINTER(FstxJoinSrc)),
+        ("n_srcs", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
+    ]
+
+
 class FstxConvertDesc(ctypes.Structure):
     _fields_ = [
         ("dst", ctypes.c_void_p),
@@ -162,6 +174,8 @@ _SIGNATURES = {
     "fstx_join_copy": (
         ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.POINTER(FstxJoinSrc), ctypes.c_uint32,
                        ctypes.c_void_p]),
+    "fstx_join_copy_batch": (
+        ctypes.c_int, [ctypes.POINTER(FstxJoinDesc), ctypes.c_uint32, ctypes.c_void_p]),
     "fstx_convert_batch": (
         ctypes.c_int, [ctypes.POINTER(FstxConvertDesc), ctypes.c_uint32, ctypes.c_void_p]),
 }
@@ -328,11 +342,20 @@ def slice_copy(dst: int, src: int, outer: int, seg_bytes: int, src_pitch: int, s
 
 
 def slice_copy_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:
-    """``jobs`` = (dst, src, outer, seg_bytes, src_pitch) tuples; any count."""
-    for i in range(0, len(jobs), FSTX_BATCH_MAX):
-        part = jobs[i : i + FSTX_BATCH_MAX]
-        arr = (FstxSliceDesc * len(part))(*[FstxSliceDesc(*j) for j in part])
-        _check("fstx_slice_copy_batch", lib().fstx_slice_copy_batch(arr, len(part), stream))
+    """``jobs`` = (dst, src, outer, seg_bytes, src_pitch) tuples; any count.
+
+    The descriptors travel as one flat array of 64-bit words (an ``fstx_slice_desc`` is five of
+    them), which costs a fraction of building a ctypes structure per job."""
+    n = len(jobs)
+    if n == 0:
+        return
+    flat = array.array("Q", [v for job in jobs for v in job])
+    base, _ = flat.buffer_info()
+    step = 5 * 8
+    fn = lib().fstx_slice_copy_batch
+    for i in range(0, n, FSTX_BATCH_MAX):
+        count = min(FSTX_BATCH_MAX, n - i)
+        _check("fstx_slice_copy_batch", fn(ctypes.cast(base + i * step, ctypes.POINTER(FstxSliceDesc)), count, stream))
 
 
 def slice_copy2d_batch(jobs: Sequence[Tuple[int, int, int, int, int, int]], stream: int = 0) -> None:
@@ -356,6 +379,22 @@ def join_copy(dst: int, rows: int, srcs: Sequence[Tuple[int, int, int]], stream:
         arr = (FstxJoinSrc * len(part))(*[FstxJoinSrc(*s) for s in part])
         _check("fstx_join_copy", lib().fstx_join_copy(at, pitch, rows, arr, len(part), stream))
         at += sum(s[1] for s in part)
+
+
+def join_copy_batch(joins: Sequence[Tuple[int, int, Sequence[Tuple[int, int, int]]]], stream: int = 0) -> None:
+    """``joins`` = (dst, rows, [(src, seg_bytes, src_pitch), ...]) with dense destinations and at
+    most ``FSTX_JOIN_MAX`` sources each; any count, as few launches as the kernel's tables allow."""
+    if not joins:
+        return
+    flat = array.array("Q", [v for _, _, srcs in joins for s in srcs for v in s])
+    base, _ = flat.buffer_info()
+    descs = (FstxJoinDesc * len(joins))()
+    at = 0
+    for d, (dst, rows, srcs) in zip(descs, joins):
+        d.dst, d.dst_pitch, d.rows, d.n_srcs = dst, 0, rows, len(srcs)
+        d.srcs = ctypes.cast(base + at * 24, ctypes.POINTER(FstxJoinSrc))
+        at += len(srcs)
+    _check("fstx_join_copy_batch", lib().fstx_join_copy_batch(descs, len(joins), stream))
 
 
 def convert_batch(jobs: Sequence[Tuple[int, int, int, int, int]], stream: int = 0) -> None:

@@ -856,8 +856,12 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
     return n_dense ? fstx_slice_copy_batch(dense, n_dense, stream) : 0;
 }
 
-extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,
-                              void *stream) {
+namespace {
+
+// one join into `gather`, or, when some block is narrower than the gather kernel takes, every
+// block on its own into its columns of the joined rows (small-unit kernel)
+int add_join(GatherBatch &gather, void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,
+             void *stream) {
     if (n == 0 || rows == 0) return 0;
     if (!dst || !srcs) return -FSTX_E_INVAL;
     if (n > FSTX_JOIN_MAX) return -FSTX_E_TOO_MANY;
@@ -871,12 +875,8 @@ extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, cons
     if (row_bytes == 0) return 0;
     if (dst_pitch == 0) dst_pitch = row_bytes;
     if (dst_pitch < row_bytes) return -FSTX_E_INVAL;
-    if (fstx_internal::gather_mode() != 0 && GatherBatch::takes(dst_pitch, rows, srcs, n)) {
-        GatherBatch gather(stream);
-        int rc = gather.add(dst, dst_pitch, rows, srcs, n);
-        return rc < 0 ? rc : gather.flush();
-    }
-    // some block is narrower than 16 bytes: every block on its own into its columns of the joined rows
+    if (fstx_internal::gather_mode() != 0 && GatherBatch::takes(dst_pitch, rows, srcs, n))
+        return gather.add(dst, dst_pitch, rows, srcs, n);
     fstx_slice2d_desc each[FSTX_JOIN_MAX];
     uint32_t m = 0;
     uint64_t col = 0;
@@ -887,6 +887,26 @@ extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, cons
         col += s.seg_bytes;
     }
     return fstx_slice_copy2d_batch(each, m, stream);
+}
+
+} // namespace
+
+extern "C" int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,
+                              void *stream) {
+    GatherBatch gather(stream);
+    int rc = add_join(gather, dst, dst_pitch, rows, srcs, n, stream);
+    return rc < 0 ? rc : gather.flush();
+}
+
+extern "C" int fstx_join_copy_batch(const fstx_join_desc *joins, uint32_t n, void *stream) {
+    if (n == 0) return 0;
+    if (!joins) return -FSTX_E_INVAL;
+    GatherBatch gather(stream);
+    for (uint32_t i = 0; i < n; ++i) {
+        int rc = add_join(gather, joins[i].dst, joins[i].dst_pitch, joins[i].rows, joins[i].srcs, joins[i].n_srcs, stream);
+        if (rc < 0) return rc;
+    }
+    return gather.flush();
 }
 
 extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, void *stream) {

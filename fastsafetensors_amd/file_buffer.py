@@ -142,6 +142,30 @@ class FilesBufferOnDevice:
             self._mark_used(*self._get_rank_lidx(name), name)
         return out.to(device=device, dtype=dtype)
 
+    def get_multi_cols_many(
+        self, groups: List[List[str]], dim: int, device: Optional[Device] = None, dtype: DType = DType.AUTO
+    ) -> List[TensorBase]:
+        """``get_multi_cols`` for many groups in one call -- the q/k/v and gate/up packing of every
+        layer, say -- with the copies of all groups batched into a few launches and the results
+        in one allocation per file.  (The reference has one call per group,
+        ``file_buffer.py:193-236``; the result of each group is the same.)"""
+        outs: List[Optional[TensorBase]] = [None] * len(groups)
+        by_file: Dict[Tuple[int, int], List[int]] = {}
+        for i, names in enumerate(groups):
+            where = {self._get_rank_lidx(n) for n in names}
+            if len(where) == 1:
+                by_file.setdefault(next(iter(where)), []).append(i)
+            else:  # a group that spans files: the one-group path joins the parts
+                outs[i] = self.get_multi_cols(names, dim, device, dtype)
+        for (rank, lidx), idx in sorted(by_file.items()):
+            made = self.rank_loaders[rank][lidx].shuffle_multi_cols_many(self.pg, [groups[i] for i in idx], dim)
+            for i, t in zip(idx, made):
+                outs[i] = t.to(device=device, dtype=dtype)
+        for i in (i for idx in by_file.values() for i in idx):
+            for name in groups[i]:
+                self._mark_used(*self._get_rank_lidx(name), name)
+        return outs  # type: ignore[return-value]
+
     def as_dict(self, tensor_shard_dim: "OrderedDict[str, int]") -> Dict[str, TensorBase]:
         """``{name: dim}`` -> ``{name: tensor}`` with the rule of ``get_sharded``."""
         out: Dict[str, TensorBase] = {}

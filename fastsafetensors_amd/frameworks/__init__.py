@@ -132,6 +132,12 @@ class FrameworkOpBase(ABC):
         tensor by a single batched copy; ``None`` when the backend cannot place them directly."""
         return None
 
+    def extract_shards_joined_many(
+        self, groups: List[List[Tuple[TensorBase, Any]]], dim: int, rank: int, world: int
+    ) -> Optional[List[TensorBase]]:
+        """``extract_shards_joined`` for many groups with batched copies; ``None`` when unsupported."""
+        return None
+
     def get_storage_shape(
         self, dtype: DType, shape: List[int], strides: List[int]
     ) -> Tuple[List[int], List[int]]:

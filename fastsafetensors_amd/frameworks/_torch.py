@@ -337,27 +337,71 @@ class TorchOp(FrameworkOpBase):
     def extract_shards(
         self, items: List[Tuple[TorchTensor, TensorFrame, int]], rank: int, world: int
     ) -> List[TorchTensor]:
-        """``extract_shard`` for many tensors with batched launches; ``dim == -1``
-        asks for a private copy of the whole tensor."""
-        outs: List[TorchTensor] = []
-        jobs = []
-        stream = None
+        """``extract_shard`` for many tensors at once; ``dim == -1`` asks for a private copy of
+        the whole tensor.
+
+        Built for hundreds of tensors per call (``as_dict`` of a checkpoint file): the copy
+        geometry of all of them goes to the library as one table and leaves as a handful of
+        batched launches *before* any result tensor exists; the results are views of ONE
+        allocation per element type (every block on a 128-byte boundary), made while the GPU is
+        already copying.  The returned tensors of one call therefore share their storage, as the
+        tensors of a file share its buffer."""
+        if not items:
+            return []
+        if not all(src.real_tensor.is_cuda for src, _, _ in items):
+            raise RuntimeError("extract_shards needs tensors in GPU memory (no CPU path exists)")
+        device = items[0][0].real_tensor.device
+        plans = []   # (dtype, native shape, element offset within its dtype's allocation)
+        rows = []    # per copy: [destination byte offset, source address, outer, seg, pitch, index of its dtype]
+        totals: Dict[torch.dtype, int] = {}
+        order: List[torch.dtype] = []
         for src, frame, dim in items:
-            if dim == -1:
-                nbytes = src.real_tensor.numel() * src.real_tensor.element_size()
-                out_shape, outer, seg, pitch, first = list(frame.shape), 1, nbytes, nbytes, 0
+            t = src.real_tensor
+            tdt = t.dtype
+            isz = t.element_size()
+            shape = frame.shape
+            nd = len(shape)
+            if dtype_size(src.dtype) < 1.0 or nd > 2 or dim >= nd or dim < -1:
+                # packed sub-byte types, higher ranks, bad dims: the general (slower) arithmetic
+                if dim == -1:
+                    out_shape, outer, seg, pitch, first = list(t.shape), 1, t.numel() * isz, t.numel() * isz, 0
+                else:
+                    st_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world, src.dtype)
+                    out_shape = self.get_native_shape(src.dtype, st_shape)
+            elif dim == -1 or nd == 0:
+                n = t.numel() * isz
+                out_shape, outer, seg, pitch, first = list(t.shape), 1, n, n, 0
             else:
-                out_shape, outer, seg, pitch, first = self.shard_geometry(frame, dim, rank, world, src.dtype)
-            dst = self.get_empty_tensor(out_shape, src.dtype, src.device)
-            outs.append(dst)
-            if outer * seg:
-                if not src.real_tensor.is_cuda:
-                    raise RuntimeError("extract_shards needs tensors in GPU memory (no CPU path exists)")
-                if stream is None:
-                    stream = torch.cuda.current_stream(src.real_tensor.device).cuda_stream
-                jobs.append((dst.data_ptr(), src.data_ptr() + first, outer, seg, pitch))
+                extent = shape[dim]
+                block = -(-extent // world)
+                lo = min(rank * block, extent)
+                mine = min(lo + block, extent) - lo
+                if nd == 1:
+                    out_shape, outer, inner = [mine], 1, isz
+                elif dim == 0:
+                    out_shape, outer, inner = [mine, shape[1]], 1, isz * shape[1]
+                else:
+                    out_shape, outer, inner = [shape[0], mine], shape[0], isz
+                seg, pitch, first = mine * inner, extent * inner, lo * inner
+            at = totals.get(tdt)
+            if at is None:
+                at = 0
+                order.append(tdt)
+            count = outer * seg // isz
+            plans.append((tdt, out_shape, at))
+            rows.append((at * isz, t.data_ptr() + first, outer, seg, pitch, tdt))
+            totals[tdt] = at + -(-count * isz // 128) * 128 // isz
+        flats = {tdt: torch.empty(max(totals[tdt], 1), dtype=tdt, device=device) for tdt in order}
+        bases = {tdt: f.data_ptr() for tdt, f in flats.items()}
+        jobs = [(bases[tdt] + off, src_at, outer, seg, pitch) for off, src_at, outer, seg, pitch, tdt in rows if outer * seg]
         if jobs:
-            _native.slice_copy_batch(jobs, stream)
+            _native.slice_copy_batch(jobs, torch.cuda.current_stream(device).cuda_stream)
+        outs: List[TorchTensor] = []
+        for (src, _, _), (tdt, out_shape, at) in zip(items, plans):
+            nd = len(out_shape)
+            strides = (out_shape[1], 1) if nd == 2 else (1,) if nd == 1 else tuple(
+                math.prod(out_shape[d + 1 :]) for d in range(nd))
+            outs.append(TorchTensor(src.device, src.dtype, torch.as_strided(flats[tdt], out_shape, strides, at)))
         return outs
 
     def extract_shards_joined(
@@ -389,6 +433,53 @@ class TorchOp(FrameworkOpBase):
                 stream,
             )
         return out
+
+    def extract_shards_joined_many(
+        self, groups: List[List[Tuple[TorchTensor, TensorFrame]]], dim: int, rank: int, world: int
+    ) -> Optional[List[TorchTensor]]:
+        """``extract_shards_joined`` for many groups at once (the q/k/v and gate/up packing of
+        every layer of a file): all results live in one allocation per element type and all
+        copies leave as a handful of batched launches."""
+        if not groups or not all(src.real_tensor.is_cuda for g in groups for src, _ in g):
+            return None
+        device = groups[0][0][0].real_tensor.device
+        plans, spans, joins = [], [], []
+        totals: Dict[torch.dtype, int] = {}
+        for items in groups:
+            geoms = [self.shard_geometry(frame, dim, rank, world, src.dtype) for src, frame in items]
+            src0 = items[0][0]
+            tdt, isz = src0.real_tensor.dtype, src0.real_tensor.element_size()
+            st_shape = list(geoms[0][0])
+            st_shape[dim] = sum(g[0][dim] for g in geoms)
+            shape = self.get_native_shape(src0.dtype, st_shape)
+            outer = geoms[0][1]
+            at = totals.get(tdt, 0)
+            nbytes = sum(g[1] * g[2] for g in geoms)
+            plans.append((src0, tdt, shape, at))
+            totals[tdt] = at + -(-nbytes // 128) * 128 // isz
+            if outer == 1:  # along the outermost dimension: the blocks are contiguous spans of the result
+                off = at * isz
+                for (src, _), (_, _o, seg, pitch, first) in zip(items, geoms):
+                    if seg:
+                        spans.append((off, src.real_tensor.data_ptr() + first, 1, seg, pitch, tdt))
+                    off += seg
+            elif nbytes:
+                joins.append((at * isz, outer, [(src.real_tensor.data_ptr() + first, seg, pitch)
+                                                for (src, _), (_, _o, seg, pitch, first) in zip(items, geoms)], tdt))
+        flats = {tdt: torch.empty(max(n, 1), dtype=tdt, device=device) for tdt, n in totals.items()}
+        bases = {tdt: f.data_ptr() for tdt, f in flats.items()}
+        stream = torch.cuda.current_stream(device).cuda_stream
+        _native.slice_copy_batch([(bases[tdt] + off, s, o, seg, pitch) for off, s, o, seg, pitch, tdt in spans], stream)
+        small = [j for j in joins if len(j[2]) <= _native.FSTX_JOIN_MAX]
+        _native.join_copy_batch([(bases[tdt] + off, rows, srcs) for off, rows, srcs, tdt in small], stream)
+        for off, rows, srcs, tdt in joins:
+            if len(srcs) > _native.FSTX_JOIN_MAX:
+                _native.join_copy(bases[tdt] + off, rows, srcs, stream)
+        outs = []
+        for src0, tdt, shape, at in plans:
+            strides = tuple(math.prod(shape[d + 1 :]) for d in range(len(shape)))
+            outs.append(TorchTensor(src0.device, src0.dtype, torch.as_strided(flats[tdt], shape, strides, at)))
+        return outs
 
     # ---- misc ------------------------------------------------------------------
     def synchronize(self, device: Device) -> None:

@@ -188,6 +188,24 @@ class LazyTensorFactory:
         pieces = self.framework.extract_shards([(h, f, dim) for h, f in zip(held, frames)], rank, world)
         return self.framework.concat_tensors(pieces, dim=dim)
 
+    def shuffle_multi_cols_many(self, pg: ProcessGroupBase, groups: List[List[str]], dim: int) -> List[TensorBase]:
+        """``shuffle_multi_cols`` for many groups of this file at once: one allocation and a
+        handful of launches for all of them."""
+        items = []
+        for names in groups:
+            frames = [self.metadata.tensors[n] for n in names]
+            ref = list(frames[0].shape)
+            for n, f in zip(names, frames):
+                for d, extent in enumerate(f.shape):
+                    if d != dim and extent != ref[d]:
+                        raise Exception(f"dim {d} mismatch: tensor {n} has {f.shape} vs. {ref} (dim={dim})")
+            items.append(list(zip([self._held(n, "shuffle_multi_cols") for n in names], frames)))
+        rank, world = (0, 1) if pg.size() == 1 else (pg.rank(), pg.size())
+        joined = self.framework.extract_shards_joined_many(items, dim, rank, world)
+        if joined is not None:
+            return joined
+        return [self.shuffle_multi_cols(pg, names, dim) for names in groups]
+
     # -- release -----------------------------------------------------------------------
     def free_dev_ptrs(self) -> None:
         self.tensors = {}

@@ -277,6 +277,20 @@ typedef struct fstx_join_src {
 int fstx_join_copy(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n,
                    void *stream);
 
+typedef struct fstx_join_desc {
+    void *dst;
+    uint64_t dst_pitch;        /* 0 = dense */
+    uint64_t rows;
+    const fstx_join_src *srcs; /* n_srcs <= FSTX_JOIN_MAX sources */
+    uint32_t n_srcs;
+    uint32_t reserved;
+} fstx_join_desc;
+
+/* Several joins at once: as many of them per launch as the kernel's tables hold (the q/k/v and
+ * gate/up packing of all layers of a file, as a caller that walks a checkpoint asks for them).
+ * Any count.  Same result as one fstx_join_copy per descriptor. */
+int fstx_join_copy_batch(const fstx_join_desc *joins, uint32_t n, void *stream);
+
 /* element types of fstx_convert_batch */
 enum fstx_elem_type {
     FSTX_F64 = 0,

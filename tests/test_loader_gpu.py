@@ -230,6 +230,51 @@ def test_as_dict_multi_cols_push_and_auto_free(small_configs):
     assert_clean()
 
 
+def test_multi_cols_many_and_shared_storage(small_configs):
+    """``get_multi_cols_many`` gives what one ``get_multi_cols`` per group gives, for joins along
+    the outermost and along an inner dimension; the tensors of one ``as_dict`` call are views of
+    one allocation, each on a 16-byte boundary, and stay valid after the file buffers are closed."""
+    files = small_configs["C4"]
+    rank, world = 1, 4
+    loader = SafeTensorsFileLoader(StubProcessGroup(rank, world), DEV)
+    loader.add_filenames({rank: files})
+    bufs = loader.copy_files_to_device()
+    bufs.auto_mem_delete = False
+    layers = sorted({int(k.split(".")[2]) for k in loader.get_keys() if k.startswith("model.layers.")})
+    for dim in (0, 1):
+        groups = []
+        for i in layers:
+            p = f"model.layers.{i}."
+            groups.append([p + f"self_attn.{x}_proj.weight" for x in "qkv"])
+            groups.append([p + f"mlp.{x}_proj.weight" for x in ("gate", "up")])
+        many = bufs.get_multi_cols_many(groups, dim=dim)
+        assert len(many) == len(groups)
+        for names, t in zip(groups, many):
+            one = bufs.get_multi_cols(names, dim=dim).get_raw()
+            assert t.get_raw().shape == one.shape and t.get_raw().data_ptr() % 16 == 0
+            assert torch.equal(t.get_raw().view(torch.int16), one.view(torch.int16)), (dim, names)
+    dims = OrderedDict((k, ck.llama_shard_dim(k)) for k in loader.get_keys())
+    out = bufs.as_dict(dims)
+    raws = {k: t.get_raw() for k, t in out.items()}
+    assert len({t.untyped_storage().data_ptr() for t in raws.values()}) <= len(files)  # one allocation per file
+    assert all(t.data_ptr() % 16 == 0 and t.is_contiguous() for t in raws.values())
+    want = {}
+    for path in files:
+        h = orc.parse_file(path)
+        for name, entry in h.tensors.items():
+            dim = dims[name]
+            if dim < 0:
+                want[name] = orc.tensor_bytes(path, h, name)
+            else:
+                want[name] = orc.shard_bytes(orc.tensor_bytes(path, h, name), entry["dtype"], entry["shape"], dim, rank, world)[0]
+    bufs.close()  # the shards are copies: they outlive the file buffers
+    loader.close()
+    for name, t in raws.items():
+        assert np.array_equal(dev_bytes(t), want[name]), name
+    del out, raws, many, t, one
+    assert_clean()
+
+
 def test_loader_reuse_and_key_order(small_configs, golden):
     loader = SafeTensorsFileLoader(SingleGroup(), DEV)
     for files in (small_configs["C3"], [golden("tiny_gpt2.safetensors")]):
