@@ -46,11 +46,23 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one launch of the roofline workload (slice_kernel, C4 column cuts, 28 tensors) moved
-# according to rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by its reading for an aligned
-# 1 GiB copy (x1.99987 and x0.99962): profiles/fstx_kernels_hbm_traffic_counters.md.  Algorithmic:
-# 1,357,905,920.
-SLICE_KERNEL_TRAFFIC_BYTES = 1_357_700_395
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "fstx_slice_kernel_c4_column_cuts_hbm_traffic.txt")
+
+
+def measured_traffic() -> dict:
+    """HBM bytes one launch of the roofline workload moved according to rocprofv3's FETCH_SIZE /
+    WRITE_SIZE counters, as written next to the counter summary under ``profiles/`` when it was
+    last refreshed (``key = value`` lines); empty when the file is missing."""
+    out = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if "=" in line and not line.lstrip().startswith("#"):
+                    k, v = line.split("=", 1)
+                    out[k.strip()] = v.strip()
+    except OSError:
+        pass
+    return out
 
 
 def log(*a):
@@ -664,6 +676,21 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         "launches_timed": len(cal_times), "avg_launch_ms": sum(cal_times) / len(cal_times),
         "bytes_per_launch": 2 * cal, "achieved_GBps": 2 * cal / 1e6 / (sum(cal_times) / len(cal_times)),
     }
+    # -- two more yardsticks for the counters, independent of this library's kernels: a kernel
+    #    that only reads 1 GiB (torch's sum) and one that only writes 1 GiB (torch's fill_)
+    ones = window[:cal].view(torch.int32)
+    for _ in range(3):
+        ones.sum()
+    rd = timed([lambda: ones.sum()] * 3)
+    for _ in range(3):
+        dst[:cal].view(torch.int32).fill_(7)
+    wr = timed([lambda: dst[:cal].view(torch.int32).fill_(7)] * 3)
+    out["counter_yardsticks"] = {
+        "read_only": {"workload": f"torch.sum over {cal} bytes of int32 (reduce_kernel: reads {cal} bytes, writes a few)",
+                      "avg_launch_ms": sum(rd) / len(rd), "bytes_read": cal},
+        "write_only": {"workload": f"torch fill_ of {cal} bytes (vectorized_elementwise_kernel FillFunctor<int>: writes {cal} bytes, reads none)",
+                       "avg_launch_ms": sum(wr) / len(wr), "bytes_written": cal},
+    }
     # -- down-cast on load: fp32 -> bf16 over 1 GiB of fp32 in 48 tensors per launch
     #    (4 bytes read + 2 written per element)
     per = cal // 4 // 48 // 64 * 64  # whole 256-byte spans, so that no cache line is shared between two jobs
@@ -1021,8 +1048,13 @@ def main() -> None:
     line["downcast_on_load"] = downcast
     if kernels:
         k = kernels["slice_extract"]
+        tr = measured_traffic()
+        # the counters belong to this workload only while its algorithmic bytes are what they were when profiled
+        same = tr.get("algorithmic_bytes_per_launch") == str(int(k["bytes_per_launch"]))
         line["roofline"] = {"bound": "hbm", "achieved": k["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                            "frac": k["achieved_GBps"] / HBM_PEAK_GBPS, "traffic": SLICE_KERNEL_TRAFFIC_BYTES,
+                            "frac": k["achieved_GBps"] / HBM_PEAK_GBPS,
+                            "traffic": int(tr["hbm_traffic_bytes_per_launch"]) if same else None,
+                            "traffic_source": os.path.relpath(TRAFFIC_FILE, ROOT) if same else "no counter profile of this workload",
                             "kernel": "slice_kernel",
                             "workload": k["workload"], "avg_launch_ms": k["avg_launch_ms"],
                             "bytes_per_launch": k["bytes_per_launch"]}
