@@ -135,3 +135,41 @@ def test_the_product_never_reaches_for_the_oracle_or_scratch_files():
         uses = any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in ast.walk(fn))
         assert uses == (fn.name == "cpu_baseline"), fn.name
     assert not any(isinstance(n, (ast.Import, ast.ImportFrom)) and "oracle" in ast.dump(n) for n in tree.body)
+
+
+def test_the_reference_side_stub_matches_the_header():
+    """INTEGRATION.md shows the ctypes stub a maintainer of the reference would add.  Its code
+    block must parse, and every ``_lib.fstx_*.argtypes`` / ``.restype`` line and the ``_Config``
+    fields in it must say what this package's own binding says (which the test above ties to
+    ``include/fstx.h``)."""
+    import ast
+
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
+    stub = next(b for b in blocks if "fastsafetensors/copier/mi355x.py" in b)
+    tree = ast.parse(stub)
+
+    def ctype(node):
+        src = ast.unparse(node)
+        return eval(src, {"ctypes": ctypes, "_Config": _native.FstxConfig})
+
+    seen = {}
+    for node in ast.walk(tree):
+        if isinstance(node, ast.Assign) and isinstance(node.targets[0], ast.Attribute):
+            target = node.targets[0]
+            if (isinstance(target.value, ast.Attribute) and isinstance(target.value.value, ast.Name)
+                    and target.value.value.id == "_lib" and target.attr in ("argtypes", "restype")):
+                seen.setdefault(target.value.attr, {})[target.attr] = ctype(node.value)
+        if isinstance(node, ast.ClassDef) and node.name == "_Config":
+            fields = next(n for n in node.body if isinstance(n, ast.Assign) and n.targets[0].id == "_fields_")
+            got = [(name, ctype_) for name, ctype_ in ctype(fields.value)]
+            assert got == list(_native.FstxConfig._fields_)
+    assert len(seen) >= 9
+    for name, sig in seen.items():
+        restype, argtypes = _native._SIGNATURES[name]
+        if "argtypes" in sig:
+            assert sig["argtypes"] == argtypes, name
+        assert sig.get("restype", ctypes.c_int) == restype, name
+    # every library function the stub calls has its signature declared
+    called = set(re.findall(r"_lib\.(fstx_\w+)\(", stub))
+    assert called <= set(seen), called - set(seen)
