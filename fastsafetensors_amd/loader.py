@@ -57,6 +57,8 @@ class BaseSafeTensorsFileLoader:
         self.meta: Dict[str, Tuple[SafeTensorsMetadata, int]] = {}
         self.frames: "OrderedDict[str, TensorFrame]" = OrderedDict()
         self.disable_cache = disable_cache
+        # headers parsed ahead of add_filenames (ParallelLoader reads the next batch's while this one loads)
+        self.parsed_ahead: Dict[str, SafeTensorsMetadata] = {}
         if not set_numa:
             kwargs.setdefault("numa_node", -1)
         self.copier_constructor: Optional[CopierConstructFunc] = create_copier_constructor(
@@ -74,6 +76,15 @@ class BaseSafeTensorsFileLoader:
         if shut is not None:
             shut()
 
+    def parse_ahead(self, paths: List[str]) -> None:
+        """Read and validate the headers of ``paths`` now, for an ``add_filenames`` that comes later.
+        Errors are left for that call to raise."""
+        for path in paths:
+            try:
+                self.parsed_ahead[path] = SafeTensorsMetadata.from_file(path, self.framework)
+            except Exception:
+                self.parsed_ahead.pop(path, None)
+
     def get_keys(self) -> List[str]:
         return list(self.frames.keys())
 
@@ -88,7 +99,7 @@ class BaseSafeTensorsFileLoader:
                 if turn >= len(paths):
                     continue
                 path = paths[turn]
-                metadata = SafeTensorsMetadata.from_file(path, self.framework)
+                metadata = self.parsed_ahead.pop(path, None) or SafeTensorsMetadata.from_file(path, self.framework)
                 self.meta[path] = (metadata, rank)
                 self.frames.update(metadata.tensors)
                 if rank == self.pg.rank():

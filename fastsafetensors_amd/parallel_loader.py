@@ -114,7 +114,17 @@ class PipelineParallel:
                 if self.stop_event.is_set():
                     self._resident.release()
                     return
-                self._ready.put(self._load_batch(batch_id, files))
+                # the next batch's headers are read while this batch's bytes are on their way
+                ahead = None
+                if batch_id + 1 < len(self.weight_files_batches):
+                    ahead = threading.Thread(target=self.loader.parse_ahead, args=(self.weight_files_batches[batch_id + 1],),
+                                             name="fstx-headers", daemon=True)
+                    ahead.start()
+                try:
+                    self._ready.put(self._load_batch(batch_id, files))
+                finally:
+                    if ahead is not None:
+                        ahead.join()
         except BaseException as e:  # surfaces in the consumer
             self.error_info = f"Producer failed: {e}"
             self.error_event.set()
