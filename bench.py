@@ -23,11 +23,15 @@ Next to it, on the same line:
                   kernel, fp32 -> bf16).
 ``tp_extract``, ``multi_cols``, ``iterate_weights``, ``downcast_on_load``
                   the callers around the path, timed through the Python API.
-``pipeline``      measured ceilings of this box -- O_DIRECT read rate of the same
-                  files, pinned host-to-device copy rate, page-cache read rate --
-                  and the cold / warm load as fractions of min(read, H2D).
-``cpu_baseline``  the reference's device="cpu" nogds path on the host cores: its
-                  own C++ reader when ``oracle/_ref`` is built, else the C
+``cold``, ``warm`` the loads next to their ceiling: the same engine with one stage
+                  left out (reads only, measured cold around every cold step;
+                  ring -> HBM copies only), ``roofline_GBps`` = the smaller of the two.
+``pipeline``      those legs, a plain O_DIRECT reader and torch's pinned copy for the
+                  record, and a cold load with adaptive read depth.
+``small_checkpoints``
+                  configs C1 and C2 cold, warm, and warm with the reader held.
+``cpu_baseline``  the reference's device="cpu" nogds path on the host cores, cold and
+                  warm: its own C++ reader when ``oracle/_ref`` is built, else the C
                   restatement in ``oracle/``.
 """
 import argparse

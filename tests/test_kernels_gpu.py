@@ -431,7 +431,7 @@ def test_entry_points_can_be_captured_in_a_graph(dev):
     the sources were changed by eager work, each compared with an eager run."""
     rows, cols = 512, 4096
     a = torch.randint(-3000, 3000, (rows, cols), dtype=torch.int16, device=dev)
-    b = torch.randint(-3000, 3000, (rows, cols + 6), dtype=torch.int16, device=dev)  # odd pitch: LDS kernel
+    b = torch.randint(-3000, 3000, (rows, cols + 6), dtype=torch.int16, device=dev)  # odd pitch: gather kernel
     f = torch.randn(rows * cols, dtype=torch.float32, device=dev)
     cut_a = torch.empty((rows, cols // 4), dtype=torch.int16, device=dev)
     cut_b = torch.empty((rows, 1001), dtype=torch.int16, device=dev)
