@@ -39,5 +39,6 @@ GOLDEN_FILES = [
     "misaligned_header.safetensors",
     "mixed_fp8.safetensors",
     "odd_bytes.safetensors",
+    "empty_at_odd.safetensors",
     "f4.safetensors",
 ]

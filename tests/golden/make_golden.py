@@ -31,6 +31,9 @@ expected values instead of trusting the files:
 ``odd_bytes.safetensors``
     U8 tensors of 3, 5 and 33 bytes in front of I16/F32 tensors, written in that
     order (not the stock order), so that wider tensors start at odd addresses.
+``empty_at_odd.safetensors``
+    Zero-byte F32 ``[0, 4]``, I64 ``[0]`` and F16 ``[3, 0]`` tensors whose offsets (3, 3 and 20)
+    are not multiples of their element sizes, between U8 / F16 tensors that hold data.
 """
 import os
 import sys
@@ -100,6 +103,18 @@ def odd_bytes_items():
     ]
 
 
+def empty_at_odd_items():
+    return [
+        ("u3", DType.U8, [3], bytes(range(3))),
+        ("e32", DType.F32, [0, 4], b""),
+        ("e64", DType.I64, [0], b""),
+        ("h", DType.F16, [2, 4], raw(torch.arange(8, dtype=torch.float16) - 2)),
+        ("u1", DType.U8, [1], b"\x7f"),
+        ("e16", DType.F16, [3, 0], b""),
+        ("tail", DType.U8, [4], bytes(range(200, 204))),
+    ]
+
+
 def main():
     save_file(tiny_gpt2_tensors(), os.path.join(HERE, "tiny_gpt2.safetensors"), metadata={"fst": "tiny-gpt2"})
     tiny = tiny_gpt2_tensors()
@@ -107,6 +122,7 @@ def main():
     write_raw(os.path.join(HERE, "misaligned_header.safetensors"), items, {"fst": "misaligned"}, 2)
     write_raw(os.path.join(HERE, "mixed_fp8.safetensors"), mixed_fp8_items(), {"fst": "mixed"}, 0)
     write_raw(os.path.join(HERE, "odd_bytes.safetensors"), odd_bytes_items(), None, 5)
+    write_raw(os.path.join(HERE, "empty_at_odd.safetensors"), empty_at_odd_items(), None, 3)
     u8 = torch.arange(64, dtype=torch.uint8).reshape(8, 8)
     save_file({"a": u8.view(torch.float4_e2m1fn_x2)}, os.path.join(HERE, "f4.safetensors"), metadata={"fst": "sample"})
     for name in sorted(os.listdir(HERE)):
