@@ -76,6 +76,32 @@ constexpr uint32_t kVec = 16;
 constexpr uint32_t kTile = kLanes * kVec; // destination bytes per wavefront
 constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two segments
 
+// Tile order for jobs whose neighbouring tiles share cache lines (a tile = the 1 KiB a wavefront
+// writes; the copy kernels use the same order).  Workgroups reach the eight dies round-robin
+// (workgroup b runs on die b % 8) and every die has its own L2, so in dispatch order the two
+// tiles either side of a shared line would sit on different dies and the line would be fetched
+// from HBM twice, or a destination line written in two parts.  The tiles are therefore dealt out
+// in chunks of 8 x 256: within a chunk die d takes tiles [256 d, 256 d + 256) one after the
+// other, so shared lines are found in that die's L2, while all dies together still sweep one
+// 2 MiB window of the job at a time -- what keeps the memory channels evenly loaded and the dies
+// in step (one contiguous eighth of the job per die measured up to 10 % slower on jobs of
+// 100 MB, and 20 % slower when the eighths alias on the channels).  The last, partial chunk is
+// dealt out in eighths.  A job takes ceil(n_tiles / 8) * 8 workgroups; false = an idle one.
+constexpr uint32_t kDies = 8;
+constexpr uint32_t kRunLog2 = 8;
+FSTX_HD bool tile_for_die(uint32_t lb, uint32_t n_tiles, uint32_t &tile) {
+    constexpr uint32_t chunk = kDies << kRunLog2;
+    const uint32_t full = n_tiles & ~(chunk - 1);
+    if (lb < full) {
+        tile = (lb & ~(chunk - 1)) | ((lb & (kDies - 1)) << kRunLog2) | ((lb / kDies) & ((1u << kRunLog2) - 1));
+        return true;
+    }
+    const uint32_t per_die = (n_tiles - full + kDies - 1) / kDies;
+    const uint32_t l = lb - full, turn = l / kDies;
+    tile = full + (l % kDies) * per_die + turn;
+    return turn < per_die && tile < n_tiles;
+}
+
 // bytes [m, m + 16) of the 32 bytes lo:hi, m in 0..15.  Written with 64-bit shifts and two-way
 // selects only: a chain of four-way selects over the eight dwords is turned back into an
 // indexed array by the compiler, and that array lands in scratch memory.

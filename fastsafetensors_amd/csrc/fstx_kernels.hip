@@ -141,6 +141,8 @@ inline uint64_t plan_grid(Table &t, const uint64_t *blocks_of, uint32_t n, uint3
     return granule << gl;
 }
 
+using fstx_gather::tile_for_die;
+
 // ------------------------------------------------------------- realign copy
 
 // bytes [4*Q + r, 4*Q + r + 16) of the 32-byte pair (lo, hi); r in 0..3
@@ -186,29 +188,25 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     v4u *dstv = reinterpret_cast<v4u *>(job.dst + head);
     const char *s = job.src + head;
     const uint32_t m = (uint32_t)(uintptr_t)s & (kVecBytes - 1);
-    // Workgroups go round-robin over the eight dies, each with its own L2.  Whenever the
-    // 1 KiB spans of neighbouring wavefronts share a cache line (source or destination not
-    // on a 128-byte boundary) or a source vector (source shifted), give each die one
-    // contiguous eighth of the job: the shared line is then fetched from HBM once and
-    // found in that die's L2 the second time, and a destination line is completed within
-    // one L2 (with neighbours on different dies it is fetched, or partially written, twice).
-    const uint64_t nblocks = (nvec + kBlock - 1) / kBlock;
-    const uint64_t per_die = (nblocks + kXcds - 1) / kXcds;
-    const uint64_t turn = lb / kXcds;
-    const uint64_t j_by_die = ((lb % kXcds) * per_die + turn) * kBlock + threadIdx.x;
+    // Whenever the 1 KiB spans of neighbouring wavefronts share a cache line (source or
+    // destination not on a 128-byte boundary) or a source vector (source shifted), neighbours
+    // run on the same die (tile_for_die).
+    uint32_t tile;
+    const bool tile_live = tile_for_die(lb, (uint32_t)((nvec + kBlock - 1) / kBlock), tile);
+    const uint64_t j_by_die = (uint64_t)tile * kBlock + threadIdx.x;
     if (m == 0) {
         // source vectors are aligned: a plain streaming copy; in dispatch order when both
         // sides sit on cache-line boundaries
         const bool by_die = ((((uintptr_t)s) | (uintptr_t)dstv) & 127) != 0;
         const uint64_t j = by_die ? j_by_die : (uint64_t)lb * kBlock + threadIdx.x;
         const v4u *srcv = reinterpret_cast<const v4u *>(s);
-        if ((!by_die || turn < per_die) && j < nvec) {
+        if ((!by_die || tile_live) && j < nvec) {
             st_stream(ld_stream(srcv + j), dstv + j);
         }
         return;
     }
     const uint64_t j = j_by_die;
-    const bool live = turn < per_die && j < nvec; // idle workgroups pad a job to whole eighths and granules
+    const bool live = tile_live && j < nvec; // idle workgroups pad a job to a multiple of eight and to granules
     // Source vectors are loaded at their natural 16-byte alignment; output vector j
     // is bytes [m, m+16) of aligned vectors j and j+1.  Every lane loads vector j
     // once and takes vector j+1 from its right-hand neighbour in the wavefront;
@@ -257,17 +255,15 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     const SliceJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
     // in dispatch order when every segment starts on a cache-line boundary on both sides,
-    // else one contiguous eighth of the job per die (see realign_kernel)
+    // else neighbours on the same die (tile_for_die)
     uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
 #ifndef FSTX_SLICE_NO_REMAP
     const uint32_t ulog = (uint32_t)(job.pitch_unit >> 56);
     const uint64_t seg_bytes = (uint64_t)job.seg_units << ulog;
     if ((((uintptr_t)job.dst | (uintptr_t)job.src | job.pitch_unit | seg_bytes) & 127) != 0) {
-        const uint32_t nblocks = (job.total_units + kBlock - 1) / kBlock;
-        const uint32_t per_die = (nblocks + kXcds - 1) / kXcds;
-        const uint32_t turn = lb / kXcds;
-        if (turn >= per_die) return;
-        u64 = ((uint64_t)(lb % kXcds) * per_die + turn) * kBlock + threadIdx.x;
+        uint32_t tile;
+        if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
+        u64 = (uint64_t)tile * kBlock + threadIdx.x;
     }
 #endif
     if (u64 >= job.total_units) return; // also retires the idle workgroups of a job's last granule
@@ -359,15 +355,12 @@ __global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2,
     const uint32_t ji = find_job(t, granule_log2, b);
     const fstx_gather::Job job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
-    // neighbouring tiles share the cache lines their common border cuts through: one contiguous
-    // eighth of the job per die (workgroup b runs on die b % 8), so that the shared line is found
-    // in that die's L2 and a destination line is completed within one L2
-    // (in dispatch order when everything sits on cache-line boundaries and nothing is shared)
+    // neighbouring tiles share the cache lines their common border cuts through: neighbours on
+    // the same die (tile_for_die); in dispatch order when everything sits on cache-line
+    // boundaries and nothing is shared
     const uint32_t n_tiles = (job.nvec + fstx_gather::kLanes - 1) / fstx_gather::kLanes;
-    const uint32_t per_die = (n_tiles + kXcds - 1) / kXcds;
-    const uint32_t turn = lb / kXcds;
-    const uint32_t tile = job.by_die ? (lb % kXcds) * per_die + turn : lb;
-    if ((job.by_die && turn >= per_die) || tile >= n_tiles) return; // idle padding of the last eighth and granule
+    uint32_t tile = lb;
+    if (job.by_die ? !tile_for_die(lb, n_tiles, tile) : tile >= n_tiles) return; // idle padding of the job's grid
     GatherMem mem;
     fstx_gather::gather_lane<kMulti, kPitched>(job, t.more, tile, threadIdx.x, mem);
 }

@@ -96,16 +96,32 @@ extern "C" int64_t fstx_gather_sim(char *dst, uint64_t dst_capacity_before, uint
     const uint64_t tiles = tiles_of(jb);
     // the leanest variant the job allows, as the library picks it (general = 1 forces the full one)
     const bool multi = n > 1 || general, pitched = dst_pitch != col || general;
-    for (uint64_t t = 0; t < tiles; ++t)
+    // workgroup by workgroup in the order the kernel deals tiles out to the dies; a tile that is
+    // skipped or visited twice shows up as payload bytes written never or twice
+    for (uint64_t lb = 0; lb < (tiles + kDies - 1) / kDies * kDies; ++lb) {
+        uint32_t t;
+        if (!tile_for_die((uint32_t)lb, (uint32_t)tiles, t)) continue;
         for (uint32_t lane = 0; lane < kLanes; ++lane) {
             if (multi && pitched) gather_lane<true, true>(jb, more.data(), (uint32_t)t, lane, mem);
             else if (multi) gather_lane<true, false>(jb, more.data(), (uint32_t)t, lane, mem);
             else if (pitched) gather_lane<false, true>(jb, more.data(), (uint32_t)t, lane, mem);
             else gather_lane<false, false>(jb, more.data(), (uint32_t)t, lane, mem);
         }
+    }
     int64_t bad = mem.errors;
     for (uint64_t r = 0; r < rows; ++r)
         for (uint64_t c = 0; c < col; ++c)
             if (written[r * dst_pitch + c] != 1) ++bad;
     return bad;
+}
+
+// The tile a workgroup takes (tile_for_die), for all workgroups of a job of n_tiles tiles:
+// out[lb] = tile, or 0xffffffff for an idle workgroup.  Returns the number of workgroups.
+extern "C" uint64_t fstx_tile_order_sim(uint32_t n_tiles, uint32_t *out) {
+    const uint64_t groups = ((uint64_t)n_tiles + kDies - 1) / kDies * kDies;
+    for (uint64_t lb = 0; lb < groups; ++lb) {
+        uint32_t t = 0;
+        out[lb] = tile_for_die((uint32_t)lb, n_tiles, t) ? t : 0xffffffffu;
+    }
+    return groups;
 }

@@ -31,6 +31,8 @@ def sim():
     lib.fstx_gather_sim.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64,
                                     ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_uint64),
                                     ctypes.POINTER(ctypes.c_uint64), ctypes.c_uint32, ctypes.c_int]
+    lib.fstx_tile_order_sim.restype = ctypes.c_uint64
+    lib.fstx_tile_order_sim.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
     return lib
 
 
@@ -124,6 +126,38 @@ def test_random_geometries(sim):
         mis = [int(x) for x in rng.integers(0, 16, n)]
         bad, same = run_case(sim, rng, rows, segs, pitches, mis, int(rng.integers(0, 16)), gap)
         assert bad == 0 and same, (trial, segs, pitches, rows, gap, mis, bad)
+
+
+@pytest.mark.parametrize("n_tiles", [1, 7, 8, 9, 255, 2047, 2048, 2049, 2056, 4095, 4096, 6000, 3 * 2048 + 1, 100_003])
+def test_tile_order_visits_every_tile_once_and_keeps_neighbours_on_a_die(sim, n_tiles):
+    out = np.empty((n_tiles + 7) // 8 * 8, dtype=np.uint32)
+    groups = sim.fstx_tile_order_sim(n_tiles, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
+    assert groups == out.size
+    live = out[out != 0xFFFFFFFF]
+    assert live.size == n_tiles and np.array_equal(np.sort(live), np.arange(n_tiles, dtype=np.uint32))
+    # workgroup b runs on die b % 8: a die's tiles come in runs of consecutive tiles (256 long in whole
+    # chunks), in ascending order, so a line shared by two neighbouring tiles is used twice by one die
+    die_of = np.empty(n_tiles, dtype=np.int64)
+    idx = np.nonzero(out != 0xFFFFFFFF)[0]
+    die_of[out[idx]] = idx % 8
+    changes = int(np.count_nonzero(np.diff(die_of)))
+    assert changes <= 8 * (n_tiles // 2048 + 1)
+    for d in range(8):
+        mine = out[d::8]
+        mine = mine[mine != 0xFFFFFFFF].astype(np.int64)
+        assert np.all(np.diff(mine) > 0)
+    # all dies work inside one window of 2048 tiles at a time
+    full = n_tiles // 2048 * 2048
+    assert np.array_equal(out[:full] // 2048, np.arange(full) // 2048)
+
+
+def test_a_job_of_several_chunks(sim):
+    rng = np.random.default_rng(15)
+    # 2046-byte segments, 2700 rows: 5.5 MB = 5395 tiles, two whole chunks and a partial one
+    bad, same = run_case(sim, rng, 2700, [2046], [8180], [6], 3, 0)
+    assert bad == 0 and same
+    bad, same = run_case(sim, rng, 900, [2046, 1022, 3000], [8180, 4090, 3001], [1, 2, 3], 5, 0)
+    assert bad == 0 and same
 
 
 def test_shapes_outside_the_kernels_domain_are_refused(sim):
