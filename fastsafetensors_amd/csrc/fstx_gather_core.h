@@ -198,6 +198,83 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
     return piece_from(s.src, s.pitch, s.seg, s.col, row, jb.rows);
 }
 
+// The common tile, decided once per wavefront: not the job's first or last tile, at most three
+// segments reach into it, and none of them lies in the first or last row of its source block.
+// Then every vector of the tile is whole payload made of at most two of the three segments, no
+// load can leave a source block, and a lane needs no division: the three segments are described
+// once per wavefront as spans of destination positions [pos, end) with a base such that position
+// p holds the byte at base + p; a lane picks its span by two comparisons, loads sixteen bytes at
+// base + its own position (and at the following span's base + position when its span ends inside
+// the vector), blends and stores.  Returns false for a tile, or on a pitched destination a lane,
+// that needs the general way below.
+struct Span {
+    uint32_t pos, end; // destination positions (bytes from the job's first, rows dst_pitch apart)
+    const char *base;  // position p of the span holds the byte at base + p
+};
+
+template <bool kMulti, bool kPitched, class Mem>
+FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, uint32_t lane, Mem &mem) {
+    const uint32_t n_tiles = (jb.nvec + kLanes - 1) / kLanes;
+    if (tile == 0 || tile + 1 >= n_tiles) return false;
+    const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
+    const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
+    const uint32_t t_lo = tile * kTile - head; // position of the tile's first byte
+    uint32_t row = t_lo / dst_pitch;
+    uint32_t c0 = t_lo - row * dst_pitch;
+    if (kPitched && c0 >= jb.row_bytes) { // the tile begins in the gap behind a row's payload
+        c0 = 0;
+        ++row;
+    }
+    const bool multi = kMulti && jb.nsrc > 1;
+    uint32_t k = multi ? source_of(jb, more, c0) : 0u;
+    uint32_t ks[3], rs[3];
+    FSTX_UNROLL
+    for (int x = 0; x < 3; ++x) {
+        ks[x] = k;
+        rs[x] = row;
+        if (++k == jb.nsrc) {
+            k = 0;
+            ++row;
+        }
+    }
+    if (rs[0] == 0 || rs[2] + 1 >= jb.rows) return false;
+    const Src first = {jb.src, jb.pitch, jb.seg, 0, 0};
+    Src s[3] = {first, first, first};
+    if (multi) { // all three descriptions are fetched before any is used
+        FSTX_UNROLL
+        for (int x = 0; x < 3; ++x) s[x] = src_uniform(more, jb.more0 + (ks[x] ? ks[x] : 1u) - 1);
+        FSTX_UNROLL
+        for (int x = 0; x < 3; ++x)
+            if (ks[x] == 0) s[x] = first;
+    }
+    Span sp[3];
+    FSTX_UNROLL
+    for (int x = 0; x < 3; ++x) {
+        sp[x].pos = rs[x] * dst_pitch + s[x].col;
+        sp[x].end = sp[x].pos + s[x].seg;
+        sp[x].base = s[x].src + (uint64_t)rs[x] * s[x].pitch - sp[x].pos;
+    }
+    if (t_lo + kTile > sp[2].end) return false; // a fourth segment reaches into the tile
+    // ---- per lane
+    const uint32_t q = t_lo + kVec * lane; // position of the vector's byte 0
+    const bool in_a = q < sp[0].end, in_ab = q < sp[1].end;
+    const uint32_t end1 = in_a ? sp[0].end : in_ab ? sp[1].end : sp[2].end;
+    const char *base1 = in_a ? sp[0].base : in_ab ? sp[1].base : sp[2].base;
+    const char *base2 = in_a ? sp[1].base : sp[2].base;
+    const bool has2 = end1 < q + kVec; // the span ends inside the vector (never the third span's: the tile ends before it does)
+    if (kPitched) { // gaps: a vector that begins or continues in one is only partly payload
+        const uint32_t pos1 = in_a ? sp[0].pos : in_ab ? sp[1].pos : sp[2].pos;
+        const uint32_t pos2 = in_a ? sp[1].pos : sp[2].pos;
+        if (q < pos1 || (has2 && pos2 != end1)) return false;
+    }
+    const Vec16 g1 = mem.load16_stream(base1 + q);
+    Vec16 g2 = {{0, 0, 0, 0}};
+    if (has2) g2 = mem.load16(base2 + q);
+    const uint32_t from2 = has2 ? end1 - q : kVec;
+    mem.store16(jb.dst + q, blend(g1, g2, from2, kVec - from2));
+    return true;
+}
+
 // One lane's work: vector `lane` of tile `tile` of job `jb`.
 //
 // A vector holds at most two parts (every segment is at least as long as a vector): the rest
@@ -215,6 +292,7 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
 // into dense destinations, the common case) runs the lean variant.
 template <bool kMulti, bool kPitched, class Mem>
 FSTX_HD void gather_lane(const Job &jb, const Src *more, uint32_t tile, uint32_t lane, Mem &mem) {
+    if (gather_lane_inner<kMulti, kPitched>(jb, more, tile, lane, mem)) return;
     const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
     const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
     // ---- once per wavefront (joins only): the segment at the start of the tile and the one after it
