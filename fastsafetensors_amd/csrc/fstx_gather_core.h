@@ -45,22 +45,23 @@ struct Vec16 {
     uint32_t w[4];
 };
 
-// 64 bytes: fetched with one wide scalar load.  The job's first source travels inside it, so a
-// job with one source (a slice extract) needs no second, dependent load before its data loads.
+// 64 bytes: fetched with one wide scalar load.  A job with one source (a slice extract) carries
+// it inside, so that no second, dependent load stands before its data loads; the sources of a
+// job with several sit in the launch's table.
 struct alignas(64) Job {
     char *dst;          // payload byte 0 of row 0, any alignment
     uint32_t dst_pitch; // bytes between destination rows, >= row_bytes
     uint32_t row_bytes; // payload bytes per row = sum of the sources' seg
     uint32_t rows;
-    uint16_t more0;     // sources 1 .. nsrc-1 are more[more0 .. more0 + nsrc - 1) of the launch
+    uint16_t more0;     // nsrc > 1: the sources are table[more0 .. more0 + nsrc) of the launch
     uint16_t nsrc;
     uint32_t nvec;      // vectors covering [align_down(dst, 16), last payload byte]
     uint32_t equal_seg; // != 0: every source has this seg, so column c belongs to source c / seg
-    const char *src;    // source 0: first byte of the block in row 0
-    uint64_t pitch;     //           bytes between its rows
-    uint32_t seg;       //           bytes per row, >= kMinSeg (its column is 0)
+    const char *src;    // nsrc == 1: first byte of the block in row 0
+    uint64_t pitch;     // nsrc == 1: bytes between its rows; nsrc > 1: magic_of(equal_seg), or 0
+    uint32_t seg;       // nsrc == 1: bytes per row, >= kMinSeg
     uint32_t by_die;    // != 0: neighbouring tiles share cache lines (something is not a multiple of 128 bytes)
-    uint64_t pad1;
+    uint64_t pitch_magic; // magic_of(dst_pitch)
 };
 
 struct alignas(32) Src {
@@ -100,6 +101,16 @@ FSTX_HD bool tile_for_die(uint32_t lb, uint32_t n_tiles, uint32_t &tile) {
     const uint32_t l = lb - full, turn = l / kDies;
     tile = full + (l % kDies) * per_die + turn;
     return turn < per_die && tile < n_tiles;
+}
+
+// Division of a 32-bit number by a divisor known on the host, d >= 2: floor(n / d) is the high
+// 64 bits of n * magic_of(d) -- exact for every n below 2^32, because the magic exceeds 2^64 / d
+// by less than d / 2^64 per unit of n.  Two multiplications instead of the twenty-odd
+// instructions of a division, in the part of a wavefront that runs before its first load.
+inline uint64_t magic_of(uint64_t d) { return d < 2 ? 0 : ~0ull / d + 1; }
+FSTX_HD uint32_t div_magic(uint32_t n, uint64_t magic) {
+    const uint64_t lo = (uint64_t)n * (uint32_t)magic, hi = (uint64_t)n * (uint32_t)(magic >> 32);
+    return (uint32_t)((hi + (lo >> 32)) >> 32);
 }
 
 // bytes [m, m + 16) of the 32 bytes lo:hi, m in 0..15.  Written with 64-bit shifts and two-way
@@ -172,9 +183,9 @@ FSTX_HD Src src_uniform(const Src *more, uint32_t index) {
 // the comparisons are per lane
 FSTX_HD uint32_t source_of(const Job &jb, const Src *more, uint32_t c) {
     if (jb.nsrc == 1) return 0;
-    if (jb.equal_seg) return c / jb.equal_seg;
+    if (jb.equal_seg) return div_magic(c, jb.pitch);
     uint32_t k = 0;
-    for (uint32_t i = 1; i < jb.nsrc; ++i) k += c >= src_uniform(more, jb.more0 + i - 1).col ? 1u : 0u;
+    for (uint32_t i = 1; i < jb.nsrc; ++i) k += c >= src_uniform(more, jb.more0 + i).col ? 1u : 0u;
     return k;
 }
 
@@ -192,9 +203,7 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
     if (!kMulti || jb.nsrc == 1) return piece_from(jb.src, jb.pitch, jb.seg, 0, row, jb.rows);
     if (row == near.row_a && c >= near.a.col && c - near.a.col < near.a.len) return near.a;
     if (row == near.row_b && c >= near.b.col && c - near.b.col < near.b.len) return near.b;
-    const uint32_t k = source_of(jb, more, c);
-    if (k == 0) return piece_from(jb.src, jb.pitch, jb.seg, 0, row, jb.rows);
-    const Src s = more[jb.more0 + k - 1]; // per lane
+    const Src s = more[jb.more0 + source_of(jb, more, c)]; // per lane
     return piece_from(s.src, s.pitch, s.seg, s.col, row, jb.rows);
 }
 
@@ -202,24 +211,21 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
 // segments reach into it, and none of them lies in the first or last row of its source block.
 // Then every vector of the tile is whole payload made of at most two of the three segments, no
 // load can leave a source block, and a lane needs no division: the three segments are described
-// once per wavefront as spans of destination positions [pos, end) with a base such that position
-// p holds the byte at base + p; a lane picks its span by two comparisons, loads sixteen bytes at
-// base + its own position (and at the following span's base + position when its span ends inside
-// the vector), blends and stores.  Returns false for a tile, or on a pitched destination a lane,
-// that needs the general way below.
-struct Span {
-    uint32_t pos, end; // destination positions (bytes from the job's first, rows dst_pitch apart)
-    const char *base;  // position p of the span holds the byte at base + p
-};
-
+// once per wavefront as spans of destination positions [pos, end); a lane picks its span by two
+// comparisons, loads the sixteen bytes that belong at its own position (and those of the
+// following span when its span ends inside the vector), blends and stores.  Returns false for a
+// tile, or on a pitched destination a lane, that needs the general way below.
 template <bool kMulti, bool kPitched, class Mem>
 FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, uint32_t lane, Mem &mem) {
+    // ---- once per wavefront, in scalar registers.  The scalar unit is shared by the four SIMDs
+    // of a compute unit and a tile is due every 190 cycles or so at full memory rate, so this
+    // part is kept short: no division, no 64-bit arithmetic, no copies.
     const uint32_t n_tiles = (jb.nvec + kLanes - 1) / kLanes;
     if (tile == 0 || tile + 1 >= n_tiles) return false;
     const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
     const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
     const uint32_t t_lo = tile * kTile - head; // position of the tile's first byte
-    uint32_t row = t_lo / dst_pitch;
+    uint32_t row = div_magic(t_lo, jb.pitch_magic);
     uint32_t c0 = t_lo - row * dst_pitch;
     if (kPitched && c0 >= jb.row_bytes) { // the tile begins in the gap behind a row's payload
         c0 = 0;
@@ -238,38 +244,51 @@ FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, ui
         }
     }
     if (rs[0] == 0 || rs[2] + 1 >= jb.rows) return false;
-    const Src first = {jb.src, jb.pitch, jb.seg, 0, 0};
-    Src s[3] = {first, first, first};
+    Src s[3];
     if (multi) { // all three descriptions are fetched before any is used
         FSTX_UNROLL
-        for (int x = 0; x < 3; ++x) s[x] = src_uniform(more, jb.more0 + (ks[x] ? ks[x] : 1u) - 1);
-        FSTX_UNROLL
-        for (int x = 0; x < 3; ++x)
-            if (ks[x] == 0) s[x] = first;
+        for (int x = 0; x < 3; ++x) s[x] = src_uniform(more, jb.more0 + ks[x]);
+    } else {
+        s[0] = s[1] = s[2] = Src{jb.src, jb.pitch, jb.seg, 0, 0};
     }
-    Span sp[3];
+    uint32_t pos[3], end[3];
     FSTX_UNROLL
     for (int x = 0; x < 3; ++x) {
-        sp[x].pos = rs[x] * dst_pitch + s[x].col;
-        sp[x].end = sp[x].pos + s[x].seg;
-        sp[x].base = s[x].src + (uint64_t)rs[x] * s[x].pitch - sp[x].pos;
+        pos[x] = rs[x] * dst_pitch + s[x].col;
+        end[x] = pos[x] + s[x].seg;
     }
-    if (t_lo + kTile > sp[2].end) return false; // a fourth segment reaches into the tile
-    // ---- per lane
+    if (t_lo + kTile > end[2]) return false; // a fourth segment reaches into the tile
+    // ---- per lane: which span, then the address (the vector units have time to spare)
     const uint32_t q = t_lo + kVec * lane; // position of the vector's byte 0
-    const bool in_a = q < sp[0].end, in_ab = q < sp[1].end;
-    const uint32_t end1 = in_a ? sp[0].end : in_ab ? sp[1].end : sp[2].end;
-    const char *base1 = in_a ? sp[0].base : in_ab ? sp[1].base : sp[2].base;
-    const char *base2 = in_a ? sp[1].base : sp[2].base;
+    const bool in_a = q < end[0], in_ab = q < end[1];
+    const uint32_t end1 = in_a ? end[0] : in_ab ? end[1] : end[2];
+    const uint32_t pos1 = in_a ? pos[0] : in_ab ? pos[1] : pos[2];
     const bool has2 = end1 < q + kVec; // the span ends inside the vector (never the third span's: the tile ends before it does)
-    if (kPitched) { // gaps: a vector that begins or continues in one is only partly payload
-        const uint32_t pos1 = in_a ? sp[0].pos : in_ab ? sp[1].pos : sp[2].pos;
-        const uint32_t pos2 = in_a ? sp[1].pos : sp[2].pos;
-        if (q < pos1 || (has2 && pos2 != end1)) return false;
+    const uint32_t pos2 = in_a ? pos[1] : pos[2];
+    if (kPitched && (q < pos1 || (has2 && pos2 != end1))) return false; // begins or continues in a gap: partly payload
+    Vec16 g1, g2 = {{0, 0, 0, 0}};
+    if (!kMulti) {
+        // one source: the three spans are consecutive rows, position p of span x holds the byte at
+        // base + x * step + p; two 64-bit values in scalar registers, one multiply-add per lane
+        const char *base = jb.src + (uint64_t)rs[0] * jb.pitch - pos[0];
+        const uint64_t step = jb.pitch - dst_pitch;
+        const uint32_t x = (in_a ? 0u : 1u) + (in_ab ? 0u : 1u); // arithmetic, not a select: selects of scalar pairs become branches
+        const char *base1 = base + x * step;
+        g1 = mem.load16_stream(base1 + q);
+        if (has2) g2 = mem.load16(base1 + step + q); // the next row begins end1 - q bytes into the vector
+    } else {
+        // several sources: the scalar unit already has the table to read, the address is put together per lane
+        const uint32_t row1 = in_a ? rs[0] : in_ab ? rs[1] : rs[2];
+        const char *src1 = in_a ? s[0].src : in_ab ? s[1].src : s[2].src;
+        const uint64_t pitch1 = in_a ? s[0].pitch : in_ab ? s[1].pitch : s[2].pitch;
+        g1 = mem.load16_stream(src1 + (uint64_t)row1 * pitch1 + (q - pos1));
+        if (has2) { // the following span begins end1 - q bytes into the vector: the load starts that far before its first byte
+            const uint32_t row2 = in_a ? rs[1] : rs[2];
+            const char *src2 = in_a ? s[1].src : s[2].src;
+            const uint64_t pitch2 = in_a ? s[1].pitch : s[2].pitch;
+            g2 = mem.load16(src2 + (uint64_t)row2 * pitch2 - (pos2 - q));
+        }
     }
-    const Vec16 g1 = mem.load16_stream(base1 + q);
-    Vec16 g2 = {{0, 0, 0, 0}};
-    if (has2) g2 = mem.load16(base2 + q);
     const uint32_t from2 = has2 ? end1 - q : kVec;
     mem.store16(jb.dst + q, blend(g1, g2, from2, kVec - from2));
     return true;
@@ -308,13 +327,11 @@ FSTX_HD void gather_lane(const Job &jb, const Src *more, uint32_t tile, uint32_t
         const uint32_t k = source_of(jb, more, c0);
         const uint32_t k2 = k + 1 < jb.nsrc ? k + 1 : 0u;
         near.row_b = k2 ? near.row_a : near.row_a + 1;
-        // both descriptions are fetched before either is used (source 0 travels in the job)
-        const Src sa = src_uniform(more, jb.more0 + (k ? k : 1u) - 1);
-        const Src sb = src_uniform(more, jb.more0 + (k2 ? k2 : 1u) - 1);
-        near.a = k ? piece_from(sa.src, sa.pitch, sa.seg, sa.col, near.row_a, jb.rows)
-                   : piece_from(jb.src, jb.pitch, jb.seg, 0, near.row_a, jb.rows);
-        near.b = k2 ? piece_from(sb.src, sb.pitch, sb.seg, sb.col, near.row_b, jb.rows)
-                    : piece_from(jb.src, jb.pitch, jb.seg, 0, near.row_b, jb.rows);
+        // both descriptions are fetched before either is used
+        const Src sa = src_uniform(more, jb.more0 + k);
+        const Src sb = src_uniform(more, jb.more0 + k2);
+        near.a = piece_from(sa.src, sa.pitch, sa.seg, sa.col, near.row_a, jb.rows);
+        near.b = piece_from(sb.src, sb.pitch, sb.seg, sb.col, near.row_b, jb.rows);
     }
     // ---- per lane
     const uint32_t j = tile * kLanes + lane;
@@ -397,14 +414,16 @@ inline uint64_t rows_per_job(uint64_t dst_pitch, uint64_t row_bytes) {
     return (kMaxSpan - row_bytes) / dst_pitch + 1;
 }
 
-// `first` is the job's source 0 (its col is 0); sources 1 .. nsrc-1 sit at more[more0 ..] of the launch
-inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t rows, const Src &first, uint32_t more0,
+// One source: `one` is it and more0 is unused.  Several: they sit at table[more0 .. more0 + nsrc)
+// of the launch and `one` is ignored.
+inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t rows, const Src &one, uint32_t more0,
                     uint32_t nsrc, uint64_t equal_seg, bool by_die = true) {
     const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
     const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
+    const bool single = nsrc == 1;
     return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,
-               (uint32_t)((head + span + kVec - 1) / kVec), (uint32_t)equal_seg, first.src, first.pitch, first.seg,
-               by_die ? 1u : 0u, 0};
+               (uint32_t)((head + span + kVec - 1) / kVec), (uint32_t)(single ? 0 : equal_seg), single ? one.src : nullptr,
+               single ? one.pitch : magic_of(equal_seg), single ? one.seg : 0u, by_die ? 1u : 0u, magic_of(dst_pitch)};
 }
 
 inline uint64_t tiles_of(const Job &jb) { return ((uint64_t)jb.nvec + kLanes - 1) / kLanes; }

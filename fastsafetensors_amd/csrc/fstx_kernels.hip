@@ -341,7 +341,7 @@ struct GatherMem {
     __device__ __forceinline__ void store8(char *p, unsigned char b) { st_global(b, reinterpret_cast<unsigned char *>(p)); }
 };
 
-// per launch: 32 jobs (each carries its first source), 24 further sources of joins, 1,024 granules
+// per launch: 32 jobs (one with a single source carries it), 24 sources of joins, 1,024 granules
 constexpr uint32_t kGatherJobs = 32;
 constexpr uint32_t kGatherMore = FSTX_JOIN_MAX;
 struct GatherTable : JobTable<fstx_gather::Job, kGatherJobs, 1024> {
@@ -626,13 +626,13 @@ struct GatherBatch {
             fstx_gather::Job job = fstx_gather::make_job(static_cast<char *>(dst) + row * dst_pitch, dst_pitch, row_bytes,
                                                          part, source(0, 0), 0, m, m > 1 ? equal : 0, lines_shared);
             const uint64_t need = (fstx_gather::tiles_of(job) + kXcds - 1) / kXcds * kXcds; // whole eighths
-            if (nj == kGatherJobs || ns + m - 1 > kGatherMore || tiles + need > lim.launch) {
+            if (nj == kGatherJobs || (m > 1 && ns + m > kGatherMore) || tiles + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
             job.more0 = (uint16_t)ns;
-            uint64_t col = live[0].seg_bytes;
-            for (uint32_t i = 1; i < m; ++i) {
+            uint64_t col = 0;
+            for (uint32_t i = 0; m > 1 && i < m; ++i) { // one source travels in the job itself
                 t.more[ns++] = source(i, col);
                 col += live[i].seg_bytes;
             }

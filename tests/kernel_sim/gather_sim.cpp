@@ -86,10 +86,10 @@ extern "C" int64_t fstx_gather_sim(char *dst, uint64_t dst_capacity_before, uint
     }
     if (dst_pitch == 0) dst_pitch = col;
     if (!shape_ok(dst_pitch, col, min_seg) || rows == 0 || rows > rows_per_job(dst_pitch, col)) return -1;
-    // the kernel's table holds sources 1 .. n-1; source 0 travels in the job
+    // the sources of a job with several sit in the launch's table; one source travels in the job
     const uint32_t more0 = 3; // somewhere inside a larger table
     std::vector<Src> more(more0 + n);
-    for (uint32_t i = 1; i < n; ++i) more[more0 + i - 1] = srcs[i];
+    for (uint32_t i = 0; i < n; ++i) more[more0 + i] = srcs[i];
     const Job jb = make_job(dst, dst_pitch, col, rows, srcs[0], more0, n, n > 1 ? equal : 0);
     std::vector<uint8_t> written((rows - 1) * dst_pitch + col, 0);
     SimMem mem{&jb, srcs.data(), &written, dst - dst_capacity_before, dst + dst_capacity_after};
@@ -125,3 +125,6 @@ extern "C" uint64_t fstx_tile_order_sim(uint32_t n_tiles, uint32_t *out) {
     }
     return groups;
 }
+
+// floor(n / d) by the kernel's multiply-high division, for the tests
+extern "C" uint32_t fstx_div_magic_sim(uint32_t n, uint64_t d) { return div_magic(n, magic_of(d)); }

@@ -31,6 +31,8 @@ def sim():
     lib.fstx_gather_sim.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64,
                                     ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_uint64),
                                     ctypes.POINTER(ctypes.c_uint64), ctypes.c_uint32, ctypes.c_int]
+    lib.fstx_div_magic_sim.restype = ctypes.c_uint32
+    lib.fstx_div_magic_sim.argtypes = [ctypes.c_uint32, ctypes.c_uint64]
     lib.fstx_tile_order_sim.restype = ctypes.c_uint64
     lib.fstx_tile_order_sim.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
     return lib
@@ -149,6 +151,24 @@ def test_tile_order_visits_every_tile_once_and_keeps_neighbours_on_a_die(sim, n_
     # all dies work inside one window of 2048 tiles at a time
     full = n_tiles // 2048 * 2048
     assert np.array_equal(out[:full] // 2048, np.arange(full) // 2048)
+
+
+def test_division_by_multiplication_is_exact(sim):
+    """The kernel divides positions by the row pitch and by the segment length with one multiply-high;
+    exact for every 32-bit numerator: checked at the multiples of the divisor and either side of them,
+    at the ends of the range, for small, odd, even, power-of-two and huge divisors."""
+    rng = np.random.default_rng(16)
+    ds = [2, 3, 5, 7, 16, 17, 31, 32, 33, 254, 1022, 2046, 2048, 4094, 6912, 8180, 8190, 96768, 65536, 65537,
+          (1 << 31) - 1, 1 << 31, (1 << 31) + 1, (1 << 32) - 1] + [int(x) for x in rng.integers(2, 1 << 32, 200)]
+    top = (1 << 32) - 1
+    for d in ds:
+        ns = {0, 1, d - 1, d, d + 1, top, top - 1, top // d * d, top // d * d - 1}
+        for m in rng.integers(0, top // d + 1, 40):
+            ns.update((int(m) * d - 1, int(m) * d, int(m) * d + 1))
+        ns.update(int(x) for x in rng.integers(0, 1 << 32, 40))
+        for n in ns:
+            if 0 <= n <= top:
+                assert sim.fstx_div_magic_sim(n, d) == n // d, (n, d)
 
 
 def test_a_job_of_several_chunks(sim):
