@@ -60,9 +60,13 @@ struct alignas(64) Job {
     const char *src;    // nsrc == 1: first byte of the block in row 0
     uint64_t pitch;     // nsrc == 1: bytes between its rows; nsrc > 1: magic_of(equal_seg), or 0
     uint32_t seg;       // nsrc == 1: bytes per row, >= kMinSeg
-    uint32_t by_die;    // != 0: neighbouring tiles share cache lines (something is not a multiple of 128 bytes)
-    uint64_t pitch_magic; // magic_of(dst_pitch)
+    uint32_t flags;     // kByDie, kByRows
+    uint64_t pitch_magic; // magic_of(dst_pitch); kByRows: magic_of(vectors_per_row(row_bytes))
 };
+
+// Job::flags
+constexpr uint32_t kByDie = 1;  // neighbouring tiles share cache lines (something is not a multiple of 128 bytes)
+constexpr uint32_t kByRows = 2; // vectors are counted row by row (see vectors_per_row)
 
 struct alignas(32) Src {
     const char *src; // first byte of the block in row 0
@@ -207,6 +211,18 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
     return piece_from(s.src, s.pitch, s.seg, s.col, row, jb.rows);
 }
 
+// A job's vectors are normally the 16-byte vectors of the memory between its first and its last
+// byte, gaps of a pitched destination included -- the lanes that land in a gap have nothing to
+// do.  When the gaps are a large part of that memory (a narrow column block written into a wide
+// tensor) the vectors are counted row by row instead: row r has the vectors that cover its own
+// payload, vectors_per_row of them at most, and a vector never holds bytes of two rows (the gap
+// is at least a vector wide).
+FSTX_HD uint32_t vectors_per_row(uint32_t row_bytes) { return (row_bytes + 2 * (kVec - 1)) / kVec; }
+inline bool counts_by_rows(uint64_t dst_pitch, uint64_t row_bytes) {
+    const uint64_t gap = dst_pitch - row_bytes;
+    return gap >= kVec && gap > dst_pitch / 8;
+}
+
 // The common tile, decided once per wavefront: not the job's first or last tile, at most three
 // segments reach into it, and none of them lies in the first or last row of its source block.
 // Then every vector of the tile is whole payload made of at most two of the three segments, no
@@ -220,6 +236,22 @@ FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, ui
     // ---- once per wavefront, in scalar registers.  The scalar unit is shared by the four SIMDs
     // of a compute unit and a tile is due every 190 cycles or so at full memory rate, so this
     // part is kept short: no division, no 64-bit arithmetic, no copies.
+    if (kPitched && (jb.flags & kByRows)) {
+        // vectors counted row by row, one source: a vector that lies inside a row's payload is one load
+        // inside that row's segment and one store (pitch_magic divides by the vectors per row here)
+        if (kMulti && jb.nsrc > 1) return false;
+        const uint32_t j = tile * kLanes + lane;
+        if (j >= jb.nvec) return false;
+        const uint32_t per_row = vectors_per_row(jb.row_bytes);
+        const uint32_t row = div_magic(j, jb.pitch_magic);
+        const uint32_t v = j - row * per_row;
+        char *row_dst = jb.dst + (uint64_t)row * jb.dst_pitch;
+        const uint32_t row_head = (uint32_t)((uintptr_t)row_dst & (kVec - 1));
+        const uint32_t c = kVec * v - row_head; // column of the vector's byte 0 (wraps when the row begins inside vector 0)
+        if ((v == 0 && row_head != 0) || c + kVec > jb.row_bytes) return false; // partly payload, or past the row's end
+        mem.store16(row_dst + c, mem.load16_stream(jb.src + (uint64_t)row * jb.pitch + c));
+        return true;
+    }
     const uint32_t n_tiles = (jb.nvec + kLanes - 1) / kLanes;
     if (tile == 0 || tile + 1 >= n_tiles) return false;
     const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
@@ -316,7 +348,8 @@ FSTX_HD void gather_lane(const Job &jb, const Src *more, uint32_t tile, uint32_t
     const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
     // ---- once per wavefront (joins only): the segment at the start of the tile and the one after it
     Near near = {{0, 0, nullptr, nullptr, nullptr}, {0, 0, nullptr, nullptr, nullptr}, 0, 0};
-    if (kMulti && jb.nsrc > 1) {
+    const bool by_rows = kPitched && (jb.flags & kByRows);
+    if (kMulti && jb.nsrc > 1 && !by_rows) {
         const uint32_t t_lo = tile == 0 ? 0u : tile * kTile - head;
         near.row_a = t_lo / dst_pitch;
         uint32_t c0 = t_lo - near.row_a * dst_pitch;
@@ -336,18 +369,33 @@ FSTX_HD void gather_lane(const Job &jb, const Src *more, uint32_t tile, uint32_t
     // ---- per lane
     const uint32_t j = tile * kLanes + lane;
     if (j >= jb.nvec) return;
-    char *out = jb.dst - head + (uint64_t)kVec * j;
-    // pitched position p is destination byte dst + p: row p / dst_pitch, column p % dst_pitch
-    uint32_t at = j == 0 ? head : 0u;       // vector 0 begins `head` bytes before the job does
-    const uint32_t q = kVec * j - head;     // position of the vector's byte 0 (wraps for j == 0 when head > 0)
-    uint32_t row = (q + at) / dst_pitch;
-    uint32_t c = (q + at) - row * dst_pitch;
-    if (kPitched && c >= jb.row_bytes) { // the vector begins in the gap behind a row's payload
-        at += dst_pitch - c;
-        c = 0;
-        ++row;
+    char *out;
+    uint32_t at, row, c;
+    if (by_rows) {
+        // vector v of row `row`: the 16 aligned bytes at align_down(the row's first byte, 16) + 16 v
+        const uint32_t per_row = vectors_per_row(jb.row_bytes);
+        row = j / per_row;
+        const uint32_t v = j - row * per_row;
+        char *row_dst = jb.dst + (uint64_t)row * dst_pitch;
+        const uint32_t row_head = (uint32_t)((uintptr_t)row_dst & (kVec - 1));
+        out = row_dst - row_head + kVec * v;
+        at = v == 0 ? row_head : 0u;
+        c = kVec * v - row_head + at;
+        if (c >= jb.row_bytes) return; // beyond this row's last vector
+    } else {
+        out = jb.dst - head + (uint64_t)kVec * j;
+        // pitched position p is destination byte dst + p: row p / dst_pitch, column p % dst_pitch
+        at = j == 0 ? head : 0u;            // vector 0 begins `head` bytes before the job does
+        const uint32_t q = kVec * j - head; // position of the vector's byte 0 (wraps for j == 0 when head > 0)
+        row = (q + at) / dst_pitch;
+        c = (q + at) - row * dst_pitch;
+        if (kPitched && c >= jb.row_bytes) { // the vector begins in the gap behind a row's payload
+            at += dst_pitch - c;
+            c = 0;
+            ++row;
+        }
+        if (at >= kVec || row >= jb.rows) return; // nothing of the job in this vector
     }
-    if (at >= kVec || row >= jb.rows) return; // nothing of the job in this vector
     // ---- part 1
     const Piece p1 = piece_of<kMulti>(jb, more, row, c, near);
     const uint32_t in1 = c - p1.col;
@@ -420,10 +468,13 @@ inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t 
                     uint32_t nsrc, uint64_t equal_seg, bool by_die = true) {
     const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
     const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
-    const bool single = nsrc == 1;
+    const bool single = nsrc == 1, by_rows = counts_by_rows(dst_pitch, row_bytes);
+    const uint64_t nvec = by_rows ? rows * vectors_per_row((uint32_t)row_bytes) : (head + span + kVec - 1) / kVec;
     return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,
-               (uint32_t)((head + span + kVec - 1) / kVec), (uint32_t)(single ? 0 : equal_seg), single ? one.src : nullptr,
-               single ? one.pitch : magic_of(equal_seg), single ? one.seg : 0u, by_die ? 1u : 0u, magic_of(dst_pitch)};
+               (uint32_t)nvec, (uint32_t)(single ? 0 : equal_seg), single ? one.src : nullptr,
+               single ? one.pitch : magic_of(equal_seg), single ? one.seg : 0u,
+               (by_die ? kByDie : 0u) | (by_rows ? kByRows : 0u),
+               magic_of(by_rows ? vectors_per_row((uint32_t)row_bytes) : dst_pitch)};
 }
 
 inline uint64_t tiles_of(const Job &jb) { return ((uint64_t)jb.nvec + kLanes - 1) / kLanes; }

@@ -360,7 +360,7 @@ __global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2,
     // boundaries and nothing is shared
     const uint32_t n_tiles = (job.nvec + fstx_gather::kLanes - 1) / fstx_gather::kLanes;
     uint32_t tile = lb;
-    if (job.by_die ? !tile_for_die(lb, n_tiles, tile) : tile >= n_tiles) return; // idle padding of the job's grid
+    if ((job.flags & fstx_gather::kByDie) ? !tile_for_die(lb, n_tiles, tile) : tile >= n_tiles) return; // idle padding of the job's grid
     GatherMem mem;
     fstx_gather::gather_lane<kMulti, kPitched>(job, t.more, tile, threadIdx.x, mem);
 }
@@ -818,13 +818,16 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
             continue;
         }
         const fstx_join_src one{d.src, d.seg_bytes, d.src_pitch};
-        if (mode != 0 && GatherBatch::takes(d.dst_pitch, d.outer, &one, 1)) {
+        const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
+                                             d.src_pitch | d.dst_pitch | 16u);
+        // a narrow block in a wide destination with everything on 16-byte boundaries: the plain
+        // 16-byte-unit kernel below has nothing to realign and measured faster on it
+        const bool plain = ul == 4 && fstx_gather::counts_by_rows(d.dst_pitch, d.seg_bytes);
+        if (mode != 0 && !plain && GatherBatch::takes(d.dst_pitch, d.outer, &one, 1)) {
             int rc = gather.add(d.dst, d.dst_pitch, d.outer, &one, 1);
             if (rc < 0) return rc;
             continue;
         }
-        const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
-                                             d.src_pitch | d.dst_pitch | 16u);
         const uint64_t seg_units = d.seg_bytes >> ul;
         uint64_t rows_per_job = lim.units() / seg_units;
         if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more

@@ -115,6 +115,22 @@ def test_pitched_destinations(sim):
             assert bad == 0 and same, (segs, gap, bad)
 
 
+def test_narrow_blocks_in_wide_rows(sim):
+    """Gaps that are a large part of the destination: the job's vectors are counted row by row.  Every
+    alignment of the first row, row pitches that change the alignment from row to row, blocks shorter and
+    longer than a tile, one source and several."""
+    rng = np.random.default_rng(17)
+    for segs, pitches in [([48], [200]), ([16], [16]), ([17], [90]), ([1000], [4000]), ([1024], [4096]), ([3000], [3001]),
+                          ([6912], [27648]), ([100, 28, 500], [300, 28, 777]), ([254, 254], [1018, 1018])]:
+        for gap in (16, 17, 24, 32, 100, 1001, 5000, 89856):
+            if gap <= (sum(segs) + gap) // 8:
+                continue  # such a gap keeps the position-wise count (covered above)
+            for dst_mis in (0, 1, 7, 8, 15):
+                mis = [int(x) for x in rng.integers(0, 16, len(segs))]
+                bad, same = run_case(sim, rng, int(rng.integers(1, 40)), segs, pitches, mis, dst_mis, gap)
+                assert bad == 0 and same, (segs, gap, dst_mis, bad)
+
+
 def test_random_geometries(sim):
     rng = np.random.default_rng(13)
     for trial in range(400):
