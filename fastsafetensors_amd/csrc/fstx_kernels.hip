@@ -485,19 +485,22 @@ __device__ __forceinline__ void convert_span(const ConvertJob &job, uint32_t lb)
     dst_t *dst = reinterpret_cast<dst_t *>(job.dst);
     const uint64_t first = ((uint64_t)lb * kBlock + threadIdx.x) * kPer;
     if (first >= job.n_elems) return;
-    // the store needs its natural alignment
-    const bool wide = ((uintptr_t)job.dst & (sizeof(out_t) - 1)) == 0 && first + kPer <= job.n_elems;
-    if (wide) {
+    if (first + kPer <= job.n_elems) {
         const v4u raw = *(const FSTX_GLOBAL in_t *)(src + first);
         src_t in[kPer];
         dst_t out[kPer];
         __builtin_memcpy(in, &raw, 16);
 #pragma unroll
         for (uint32_t k = 0; k < kPer; ++k) out[k] = Elem<D>::from_f32(Elem<S>::to_f32(in[k]));
-        out_t packed;
-        __builtin_memcpy(&packed, out, sizeof packed);
-        st_global(packed, reinterpret_cast<out_t *>(dst + first));
-    } else { // misaligned destination or the ragged end: element by element
+        if (((uintptr_t)job.dst & (sizeof(out_t) - 1)) == 0) { // uniform: one store at its natural alignment
+            out_t packed;
+            __builtin_memcpy(&packed, out, sizeof packed);
+            st_global(packed, reinterpret_cast<out_t *>(dst + first));
+        } else { // a destination that is only element-aligned: one store per element
+#pragma unroll
+            for (uint32_t k = 0; k < kPer; ++k) st_global(out[k], dst + first + k);
+        }
+    } else { // the ragged end: element by element
         for (uint32_t k = 0; k < kPer && first + k < job.n_elems; ++k)
             st_global(Elem<D>::from_f32(Elem<S>::to_f32(ld_global(src + first + k))), dst + first + k);
     }
@@ -508,7 +511,16 @@ __global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t granule_
     const uint32_t b = blockIdx.x;
     const uint32_t ji = find_job(t, granule_log2, b);
     const ConvertJob job = t.fetch(ji);
-    const uint32_t lb = b - t.first_block[ji];
+    uint32_t lb = b - t.first_block[ji];
+    // a job that does not begin on cache lines shares them between neighbouring workgroups:
+    // neighbours on the same die (tile_for_die), as in the copy kernels
+    if ((((uintptr_t)job.src | (uintptr_t)job.dst) & 127) != 0) {
+        const uint32_t per_block_log2 = 7 + (job.src_type < 2 ? job.src_type : 2); // 64 lanes x 16 bytes of f64 / f32 / 16-bit
+        const uint32_t n_tiles = (uint32_t)((job.n_elems + (1ull << per_block_log2) - 1) >> per_block_log2);
+        uint32_t tile;
+        if (!tile_for_die(lb, n_tiles, tile)) return;
+        lb = tile;
+    }
 #define FSTX_CONVERT(S, D) \
     case (S) * 8 + (D): convert_span<S, D>(job, lb); break;
     switch (job.src_type * 8 + job.dst_type) { // uniform across the workgroup
@@ -941,7 +953,9 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         const uint64_t piece = lim.job * per_block; // elements one job may take
         for (uint64_t done = 0; done < d.n_elems; done += piece) {
             const uint64_t len = d.n_elems - done < piece ? d.n_elems - done : piece;
-            const uint64_t need = (len + per_block - 1) / per_block;
+            uint64_t need = (len + per_block - 1) / per_block;
+            if ((((uintptr_t)(db + done * ds) | (uintptr_t)(sb + done * ss)) & 127) != 0)
+                need = (need + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
             if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
