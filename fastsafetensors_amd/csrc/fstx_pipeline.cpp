@@ -281,6 +281,7 @@ struct fstx_ctx {
     std::mutex table_mutex;
     std::map<int64_t, std::shared_ptr<FileEntry>> files;
     std::map<int64_t, std::shared_ptr<Request>> requests;
+    std::vector<fstx_dev::event_t> event_pool; // markers of finished waits, for the next ones (table_mutex)
     int64_t next_file = 1;
     int64_t next_request = 1;
 
@@ -815,15 +816,21 @@ int normalize(fstx_config &cfg) {
 }
 
 void free_parts(fstx_ctx *ctx) {
+    const uint64_t t0 = now_ns();
     for (auto &per : ctx->slots)
         for (Slot &s : per)
             if (s.ev) fstx_dev::event_destroy(s.ev);
     if (ctx->order_event) fstx_dev::event_destroy(ctx->order_event);
+    for (auto e : ctx->event_pool) fstx_dev::event_destroy(e);
+    const uint64_t t1 = now_ns();
     for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
+    const uint64_t t2 = now_ns();
     if (ctx->ring) {
         fstx_dev::host_free(ctx->ring);
         fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
     }
+    fstx_internal::debug("free_parts: events %.2f ms, streams %.2f ms, ring %.2f ms", (t1 - t0) / 1e6, (t2 - t1) / 1e6,
+                         (now_ns() - t2) / 1e6);
 }
 
 void stop_workers(fstx_ctx *ctx) {
@@ -937,14 +944,19 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 
 int fstx_ctx_destroy(fstx_ctx *ctx) {
     if (!ctx) return -FSTX_E_INVAL;
+    const uint64_t t0 = now_ns();
     stop_workers(ctx);
+    const uint64_t t1 = now_ns();
     if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->limit());
     fstx_dev::set_device(ctx->cfg.device_id);
     for (auto s : ctx->streams) fstx_dev::stream_sync(s);
     for (auto &kv : ctx->files) release_file(*kv.second);
     for (char *p : ctx->stage_free) std::free(p);
+    const uint64_t t2 = now_ns();
     free_parts(ctx);
     delete ctx;
+    fstx_internal::debug("ctx_destroy: workers joined in %.2f ms, streams idle and files closed in %.2f ms, ring, events and streams freed in %.2f ms",
+                         (t1 - t0) / 1e6, (t2 - t1) / 1e6, (now_ns() - t2) / 1e6);
     return 0;
 }
 
@@ -1123,15 +1135,63 @@ int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request) {
         std::unique_lock<std::mutex> lk(ctx->done_mutex);
         ctx->done_cv.wait(lk, [&] { return req->blocks_left.load(std::memory_order_acquire) == 0; });
     }
-    // every block is enqueued on its stream by now; wait for the copies themselves
+    bool alone; // no other request submitted and not yet waited for
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        alone = ctx->requests.empty();
+    }
+    // Every block is enqueued on its stream by now; wait for the copies themselves.  With nothing
+    // queued behind them the streams are synchronized (which also lets the runtime retire their
+    // finished commands while this thread has to wait anyway; left to pile up until the streams
+    // are destroyed, they cost milliseconds there).  A caller that queues the next files before
+    // waiting for these keeps the streams busy, and a synchronize of a stream that is being fed
+    // returned 8 ms after these copies were done: then a marker is put behind them on each stream
+    // and waited for instead.
     int64_t status = req->error.load();
-    uint64_t mask = req->stream_mask.load();
+    const uint64_t mask = req->stream_mask.load();
     fstx_dev::set_device(ctx->cfg.device_id);
-    for (size_t i = 0; i < ctx->streams.size(); ++i)
-        if (mask & (1ull << i)) {
-            int rc = fstx_dev::stream_sync(ctx->streams[i]);
-            if (rc < 0 && status == 0) status = rc;
+    if (alone) {
+        for (size_t i = 0; i < ctx->streams.size(); ++i)
+            if (mask >> i & 1) {
+                int rc = fstx_dev::stream_sync(ctx->streams[i]);
+                if (rc < 0 && status == 0) status = rc;
+            }
+        req->file->open_requests.fetch_sub(1);
+        return status < 0 ? status : (int64_t)req->length;
+    }
+    std::vector<fstx_dev::event_t> marks;
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        for (size_t i = 0; i < ctx->streams.size(); ++i)
+            if ((mask >> i & 1) && !ctx->event_pool.empty()) {
+                marks.push_back(ctx->event_pool.back());
+                ctx->event_pool.pop_back();
+            }
+    }
+    size_t m = 0;
+    std::vector<fstx_dev::event_t> used;
+    for (size_t i = 0; i < ctx->streams.size(); ++i) {
+        if (!(mask >> i & 1)) continue;
+        fstx_dev::event_t ev = nullptr;
+        if (m < marks.size()) ev = marks[m++];
+        int rc = ev ? 0 : fstx_dev::event_create(&ev);
+        if (rc == 0) {
+            used.push_back(ev);
+            rc = fstx_dev::event_record(ev, ctx->streams[i]);
         }
+        if (rc < 0) { // no marker to be had: the stream itself
+            int rs = fstx_dev::stream_sync(ctx->streams[i]);
+            if (rs < 0 && status == 0) status = rs;
+        }
+    }
+    for (fstx_dev::event_t ev : used) {
+        int rc = fstx_dev::event_sync(ev);
+        if (rc < 0 && status == 0) status = rc;
+    }
+    {
+        std::lock_guard<std::mutex> lk(ctx->table_mutex);
+        ctx->event_pool.insert(ctx->event_pool.end(), used.begin(), used.end());
+    }
     req->file->open_requests.fetch_sub(1);
     return status < 0 ? status : (int64_t)req->length;
 }

@@ -116,12 +116,23 @@ class BaseSafeTensorsFileLoader:
         The returned object owns the device memory; tensors taken from it must be
         cloned before its ``close()`` if they are to outlive it.
         """
+        return self.start_copy(dtype, use_buf_register, max_copy_block_size).finish()
+
+    def start_copy(
+        self,
+        dtype: DType = DType.AUTO,
+        use_buf_register: bool = True,
+        max_copy_block_size: int = 16 * 1024 * 1024 * 1024,
+    ) -> "PendingCopy":
+        """The first half of ``copy_files_to_device``: allocate the registered files' buffers and queue
+        their reads; ``finish()`` of the returned object waits for them.  The loader may be ``reset()``
+        and given the next files in between, so that their reads queue up behind these without the
+        transfer ever pausing (``ParallelLoader`` does)."""
         if self.copier_constructor is None:
             raise Exception("copy_files_to_device: loader is closed")
         self.framework.set_device(self.device)
-        factories: Dict[int, List[LazyTensorFactory]] = {r: [] for r in range(self.pg.size())}
+        pending = PendingCopy(self, dtype)
         idx_bits = math.ceil(math.log2(len(self.meta) + 1))
-        mine: List[LazyTensorFactory] = []
         try:
             for lidx, (path, (meta, rank)) in enumerate(sorted(self.meta.items()), start=1):
                 local = rank == self.pg.rank()
@@ -130,25 +141,49 @@ class BaseSafeTensorsFileLoader:
                     meta, self.device, rank, local, idx_bits, lidx, copier, self.framework,
                     disable_cache=self.disable_cache,
                 )
-                factories.setdefault(rank, []).append(factory)
+                pending.factories.setdefault(rank, []).append(factory)
                 factory.submit_io(use_buf_register, max_copy_block_size)
                 if local:
-                    mine.append(factory)
-            for factory in mine:
-                factory.wait_io(dtype=dtype, noalign=False)
+                    pending.mine.append(factory)
+        except Exception:
+            pending.abandon()
+            raise
+        return pending
+
+
+class PendingCopy:
+    """Files whose reads are queued (``BaseSafeTensorsFileLoader.start_copy``)."""
+
+    def __init__(self, loader: BaseSafeTensorsFileLoader, dtype: DType):
+        self.framework = loader.framework
+        self.device = loader.device
+        self.pg = loader.pg
+        self.dtype = dtype
+        self.factories: Dict[int, List[LazyTensorFactory]] = {r: [] for r in range(loader.pg.size())}
+        self.mine: List[LazyTensorFactory] = []
+
+    def finish(self) -> FilesBufferOnDevice:
+        """Wait for the reads and hand the buffers over."""
+        try:
+            for factory in self.mine:
+                factory.wait_io(dtype=self.dtype, noalign=False)
             # wait_io may have queued realign / convert kernels on this thread's stream: the
             # tensors are complete when this call returns, as after the reference's synchronous copies
             self.framework.synchronize_stream(self.device)
-            return FilesBufferOnDevice(factories, pg=self.pg, framework=self.framework)
+            return FilesBufferOnDevice(self.factories, pg=self.pg, framework=self.framework)
         except Exception:
-            # leave no arena and no in-flight read behind
-            for factory in mine:
-                try:
-                    if factory.copier is not None and hasattr(factory.copier, "_drain"):
-                        factory.copier._drain()
-                finally:
-                    factory.free_dev_ptrs()
+            self.abandon()
             raise
+
+    def abandon(self) -> None:
+        """Leave no arena and no in-flight read behind."""
+        mine, self.mine = self.mine, []
+        for factory in mine:
+            try:
+                if factory.copier is not None and hasattr(factory.copier, "_drain"):
+                    factory.copier._drain()
+            finally:
+                factory.free_dev_ptrs()
 
 
 class SafeTensorsFileLoader(BaseSafeTensorsFileLoader):

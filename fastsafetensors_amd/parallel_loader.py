@@ -90,14 +90,22 @@ class PipelineParallel:
         self.need_clone = self.pg.size() == 1
 
     # -- producer ---------------------------------------------------------------------
-    def _load_batch(self, batch_id: int, files: List[str]) -> FileBatch:
+    def _start_batch(self, batch_id: int, files: List[str]) -> Tuple[int, Any, float, float]:
+        """Headers, buffers and queued reads of one batch; ``_finish_batch`` waits for them."""
         t0 = time.perf_counter()
         # file i of a batch belongs to rank i; a stub group owns the file of the rank it reports
         self.loader.add_filenames({rank: [f] for rank, f in enumerate(files)})
         t1 = time.perf_counter()
-        fb = self.loader.copy_files_to_device()
+        try:
+            pending = self.loader.start_copy()
+        finally:
+            self.loader.reset()
+        return batch_id, pending, t0, t1
+
+    def _finish_batch(self, started: Tuple[int, Any, float, float]) -> FileBatch:
+        batch_id, pending, t0, t1 = started
+        fb = pending.finish()
         t2 = time.perf_counter()
-        self.loader.reset()
         batch = FileBatch(fb, list(fb.key_to_rank_lidx.keys()), batch_id)
         batch.add_filenames_time = (t1 - t0) * 1e3
         batch.copy_files_time = (t2 - t1) * 1e3
@@ -105,14 +113,37 @@ class PipelineParallel:
         logger.debug("batch %d loaded: %d keys, %.1f ms", batch_id, len(batch.keys), batch.load_time)
         return batch
 
+    def _load_batch(self, batch_id: int, files: List[str]) -> FileBatch:
+        return self._finish_batch(self._start_batch(batch_id, files))
+
+    def _acquire_slot(self, patience: Optional[float]) -> bool:
+        """A place among the resident batches; gives up after ``patience`` seconds (None: never) or when stopped."""
+        if patience is not None and patience <= 0:
+            return self._resident.acquire(blocking=False)
+        deadline = None if patience is None else time.perf_counter() + patience
+        while not self._resident.acquire(timeout=0.005 if patience is not None else 0.05):
+            if self.stop_event.is_set() or (deadline is not None and time.perf_counter() >= deadline):
+                return False
+        if self.stop_event.is_set():
+            self._resident.release()
+            return False
+        return True
+
     def _producer_worker(self) -> None:
+        # The reads of batch k+1 are queued before batch k is waited for whenever a place is free
+        # by then (the consumer has usually let go of batch k-1 within a few milliseconds), so the
+        # transfer streams on across the batch boundary instead of draining and starting again.
+        started: Optional[Tuple[int, Any, float, float]] = None
         try:
             for batch_id, files in enumerate(self.weight_files_batches):
-                while not self._resident.acquire(timeout=0.05):
-                    if self.stop_event.is_set():
-                        return
-                if self.stop_event.is_set():
-                    self._resident.release()
+                # (with one resident batch at most there is never a place while a batch is loading)
+                ahead_ok = self._acquire_slot(None if started is None else 0.0 if self.queue_size < 0 else 0.02)
+                if not ahead_ok and started is not None:
+                    # no place yet: hand the loaded batch over first, then wait for one
+                    self._ready.put(self._finish_batch(started))
+                    started = None
+                    ahead_ok = self._acquire_slot(None)
+                if not ahead_ok:
                     return
                 # the next batch's headers are read while this batch's bytes are on their way
                 ahead = None
@@ -121,15 +152,42 @@ class PipelineParallel:
                                              name="fstx-headers", daemon=True)
                     ahead.start()
                 try:
-                    self._ready.put(self._load_batch(batch_id, files))
+                    try:
+                        following = self._start_batch(batch_id, files)
+                    except BaseException:
+                        self._resident.release()
+                        if started is not None:
+                            # the batch before the failing one is whole: it is handed over first
+                            previous, started = started, None
+                            self._ready.put(self._finish_batch(previous))
+                        raise
+                    if started is not None:
+                        previous, started = started, following
+                        self._ready.put(self._finish_batch(previous))
+                    else:
+                        started = following
                 finally:
                     if ahead is not None:
                         ahead.join()
+            if started is not None:
+                last, started = started, None
+                self._ready.put(self._finish_batch(last))
         except BaseException as e:  # surfaces in the consumer
+            if started is not None:
+                try:
+                    started[1].abandon()
+                except Exception:
+                    pass
             self.error_info = f"Producer failed: {e}"
             self.error_event.set()
             self._ready.put(e)
             return
+        finally:
+            if started is not None and self.stop_event.is_set():
+                try:
+                    started[1].abandon()
+                except Exception:
+                    pass
         self._ready.put(None)
 
     # -- consumer ---------------------------------------------------------------------
