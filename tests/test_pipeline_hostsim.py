@@ -307,6 +307,34 @@ def test_order_after_holds_the_copies_back(sim, blob):
     sim.fstx_ctx_destroy(ctx)
 
 
+def test_wait_covers_its_own_request_while_later_ones_keep_the_streams_busy(sim, blob):
+    """A caller may queue the next file's reads before it waits for this one's: the wait returns
+    when this request's bytes are in place, neither earlier nor only when the streams run dry."""
+    import time
+    path, data = blob
+    sim.fstx_sim_set_copy_delay_us(400)
+    try:
+        ctx = make_ctx(sim, threads=4, streams=2, block=64 * 1024)
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        first = np.zeros(1_000_000, dtype=np.uint8)
+        later = np.zeros(8_000_000, dtype=np.uint8)
+        a = sim.fstx_submit_read(ctx, f, 0, first.size, first.ctypes.data, first.size, 0)
+        b = sim.fstx_submit_read(ctx, f, first.size, later.size, later.ctypes.data, later.size, 0)
+        t0 = time.perf_counter()
+        assert sim.fstx_wait_read(ctx, a) == first.size
+        t_a = time.perf_counter() - t0
+        assert np.array_equal(first, data[: first.size])       # complete the moment the wait returns
+        assert not np.array_equal(later, data[first.size : first.size + later.size])  # the later request is still on its way
+        assert sim.fstx_wait_read(ctx, b) == later.size
+        t_b = time.perf_counter() - t0
+        assert np.array_equal(later, data[first.size : first.size + later.size])
+        assert t_a < 0.6 * t_b, (t_a, t_b)
+        assert sim.fstx_file_close(ctx, f) == 0
+        assert sim.fstx_ctx_destroy(ctx) == 0
+    finally:
+        sim.fstx_sim_set_copy_delay_us(30)
+
+
 def test_direct_reads_ramp_up_and_down(sim, blob):
     """O_DIRECT runs: small first, growing fourfold to the full size, halving towards the end of
     what is queued; a ramp size at or above the full size keeps every read at full size."""

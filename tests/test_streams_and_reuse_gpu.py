@@ -248,3 +248,30 @@ def test_downcast_of_types_the_kernel_has_no_pair_for(tmp_path, layout):
     bufs.close()
     loader.close()
     assert_clean()
+
+
+def test_two_batches_of_files_in_flight(data_dir):
+    """start_copy / finish: the second batch's reads are queued before the first is waited for (what
+    ParallelLoader does between batches).  Each batch is complete when its finish() returns -- compared
+    byte for byte with the stock loader right then, while the other batch may still be on its way."""
+    cfg = ck.configs(0.05)["C3"]
+    files = [r["path"] for r in ck.write_config(cfg, os.path.join(data_dir, "two_batches"))]
+    assert len(files) >= 4
+    loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=8)
+    pending = []
+    for batch in (files[:2], files[2:4]):
+        loader.add_filenames({0: batch})
+        pending.append((batch, loader.start_copy()))
+        loader.reset()
+    for batch, p in pending:
+        bufs = p.finish()
+        for path in batch:
+            for key, want in load_file(path).items():
+                got = bufs.get_tensor(key)
+                assert np.array_equal(dev_bytes(got), want.reshape(-1).view(torch.uint8).numpy()), key
+        bufs.close()
+    # an abandoned batch leaves nothing behind
+    loader.add_filenames({0: files[:1]})
+    loader.start_copy().abandon()
+    loader.close()
+    assert_clean()
