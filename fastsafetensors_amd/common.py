@@ -287,10 +287,9 @@ class SafeTensorsMetadata:
                 "get_tensors builds views only; conversion on load is done by the copier (wait_io)"
             )
         shift = self.header_length - copy_start_offset
-        return {
-            name: self.framework.view_tensor(gbuf, shift + frame.data_offsets[0], frame, device)
-            for name, frame in self.tensors.items()
-        }
+        return self.framework.view_tensors(
+            gbuf, [(name, shift + frame.data_offsets[0], frame) for name, frame in self.tensors.items()], device
+        )
 
     def __repr__(self) -> str:
         return str({"__metadata__": self.metadata, "tensors": self.tensors})

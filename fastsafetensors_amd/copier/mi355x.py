@@ -184,13 +184,11 @@ class MI355XFileCopier(CopierInterface):
                 self._stream(),
             )
 
-        tensors: Dict[str, TensorBase] = {}
-        for name, frame in meta.tensors.items():
-            if name in placed:
-                tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
-            else:
-                tensors[name] = fw.view_tensor(arena, data_at + frame.data_offsets[0], frame, self.device)
-        return tensors
+        in_arena = [(n, data_at + f.data_offsets[0], f) for n, f in meta.tensors.items() if n not in placed]
+        views = fw.view_tensors(arena, in_arena, self.device)
+        if placed:
+            views.update(fw.view_tensors(side, [(n, placed[n], meta.tensors[n]) for n in placed], self.device))
+        return {name: views[name] for name in meta.tensors}  # in the file's order
 
     def _converted(self, gbuf: _native.DeviceBuffer, dtype: DType) -> Dict[str, TensorBase]:
         """Tensors down-cast to ``dtype`` on the GPU (``common.py:355-375`` does it with

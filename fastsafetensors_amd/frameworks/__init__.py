@@ -11,7 +11,7 @@ package hands work to its HIP library instead of DLPack capsules and
 
 from abc import ABC, abstractmethod
 from dataclasses import dataclass
-from typing import Any, List, Optional, Sequence, Tuple
+from typing import Dict, Any, List, Optional, Sequence, Tuple
 
 from ..st_types import Device, DType
 
@@ -111,6 +111,11 @@ class FrameworkOpBase(ABC):
     @abstractmethod
     def view_tensor(self, gbuf: Any, byte_offset: int, frame: Any, device: Device) -> TensorBase:
         """Zero-copy tensor over ``gbuf[byte_offset : byte_offset + frame.nbytes]``."""
+
+    def view_tensors(self, gbuf: Any, items: Any, device: Device) -> Dict[str, TensorBase]:
+        """``view_tensor`` for many ``(name, byte_offset, frame)`` over one buffer; a framework may do
+        it with less work per tensor."""
+        return {name: self.view_tensor(gbuf, off, frame, device) for name, off, frame in items}
 
     @abstractmethod
     def extract_shard(

@@ -201,3 +201,43 @@ def test_tensor_frame_getitem_follows_sequences():
         frame()["x"]
     nested = frame()[1:4][1:]  # offsets accumulate
     assert nested.offsets == [2, 0] and nested.shape == [2, m]
+
+
+@pytest.mark.parametrize("name", GOLDEN_FILES)
+def test_batched_views_equal_the_views_made_one_by_one(golden, name):
+    """``view_tensors`` (one typed view of the buffer per dtype + ``as_strided``) against ``view_tensor``
+    (slice, view, view) over a host copy of the file: same address, shape, strides, dtype and bytes for
+    every tensor -- scalars, packed fp4, empty tensors and tensors at odd offsets included."""
+    import numpy as np
+    import torch
+
+    from fastsafetensors_amd import _native
+
+    path = golden(name)
+    fwk = get_framework_op("pytorch")
+    meta = SafeTensorsMetadata.from_file(path, fwk)
+    raw = np.fromfile(path, dtype=np.uint8)[meta.header_length:]
+    arena = torch.zeros(raw.size + 16, dtype=torch.uint8)
+    arena[: raw.size] = torch.from_numpy(raw.copy())
+    buf = _native.DeviceBuffer(arena.data_ptr(), arena.numel(), True)
+    buf.keepalive = arena
+    from fastsafetensors_amd.st_types import Device
+
+    device = Device.from_str("cpu")
+    items = [(k, f.data_offsets[0], f) for k, f in meta.tensors.items()]
+    one_by_one = {}
+    for k, off, f in items:
+        try:
+            one_by_one[k] = fwk.view_tensor(buf, off, f, device).get_raw()
+        except RuntimeError:
+            one_by_one[k] = None  # torch refuses a view at an offset that is odd for the dtype (the copier realigns those)
+    aligned = [(k, off, f) for k, off, f in items if one_by_one[k] is not None]
+    batched = fwk.view_tensors(buf, aligned, device)
+    assert list(batched) == [k for k, _, _ in aligned]
+    for k, _, f in aligned:
+        a, b = one_by_one[k], batched[k].get_raw()
+        assert a.dtype == b.dtype and a.shape == b.shape and a.stride() == b.stride() and b.is_contiguous(), k
+        assert (a.numel() == 0 and b.numel() == 0) or a.data_ptr() == b.data_ptr(), k
+        assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), k
+    with pytest.raises(IndexError):
+        fwk.view_tensors(buf, [(items[0][0], arena.numel() - 1, items[0][2])], device)
