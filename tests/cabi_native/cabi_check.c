@@ -6,9 +6,11 @@
  *
  *   cabi_check FILE
  *
- * Loads FILE (any bytes) into device memory with the read pipeline in every read mode,
- * then checks the realign copy, the slice extract (dense, strided destination, joined)
- * and the fp32 -> bf16 conversion against loops on the host.  Prints "cabi_check: ok".
+ * Loads FILE (any bytes) into device memory with the read pipeline in every read mode, through
+ * a private and through a shared context, then checks the realign copy, the slice extract
+ * (dense, batched, strided destination, joined, joined in a batch) and the fp32 -> bf16
+ * conversion against loops on the host, and calls the small entry points.  Every function
+ * include/fstx.h declares is called at least once.  Prints "cabi_check: ok".
  */
 #include <stdint.h>
 #include <stdio.h>
@@ -53,8 +55,8 @@ int main(int argc, char **argv) {
     uint64_t size = (uint64_t)ftell(fp);
     fseek(fp, 0, SEEK_SET);
     CHECK(size >= 4096);
-    unsigned char *want = malloc(size), *got = malloc(size);
-    CHECK(want && got && fread(want, 1, size, fp) == size);
+    unsigned char *want = malloc(size), *got = malloc(size), *tmp = malloc(size);
+    CHECK(want && got && tmp && fread(want, 1, size, fp) == size);
     fclose(fp);
 
     CHECK(fstx_abi_version() == FSTX_ABI_VERSION);
@@ -96,6 +98,29 @@ int main(int argc, char **argv) {
     CHECK(fstx_ctx_destroy(ctx) == 0);
     CHECK(fstx_bounce_buffer_bytes() == 0);
 
+    /* ---- a shared context: two users, one ring; ordered after the null stream's work ---- */
+    {
+        fstx_ctx *a = NULL, *b = NULL;
+        CHECK(fstx_ctx_acquire(&cfg, &a) == 0 && fstx_ctx_acquire(&cfg, &b) == 0 && a == b);
+        const uint64_t ring = fstx_bounce_buffer_bytes();
+        CHECK(ring > 0);
+        CHECK(hipMemset(arena, 0x11, size + 256) == hipSuccess); /* queued on the null stream ... */
+        CHECK(fstx_ctx_order_after(a, NULL) == 0);               /* ... and the copies come after it */
+        int64_t file = fstx_file_open(b, argv[1], FSTX_READ_BUFFERED);
+        CHECK(file > 0);
+        int64_t first = fstx_submit_read(a, file, 0, size / 2, arena, size + 256, 0);
+        int64_t second = fstx_submit_read(b, file, size / 2, size - size / 2, arena, size + 256, size / 2);
+        CHECK(first > 0 && second > 0);
+        CHECK(fstx_wait_read(a, first) == (int64_t)(size / 2)); /* with the second still in flight */
+        CHECK(fstx_wait_read(b, second) == (int64_t)(size - size / 2));
+        CHECK(fstx_file_close(a, file) == 0);
+        CHECK(hipMemcpy(got, arena, size, hipMemcpyDeviceToHost) == hipSuccess && memcmp(got, want, size) == 0);
+        CHECK(fstx_ctx_release(a) == 0 && fstx_bounce_buffer_bytes() == ring); /* one user left */
+        CHECK(fstx_ctx_release(b) == 0 && fstx_bounce_buffer_bytes() == 0);
+        /* put the bytes back where the kernel checks below expect them */
+        CHECK(hipMemcpy(arena + 3, want + 10, size - 10, hipMemcpyHostToDevice) == hipSuccess);
+    }
+
     /* ---- kernels: arena + 3 holds file bytes [10, size) ---- */
     const unsigned char *src = arena + 3;
     const unsigned char *hsrc = want + 10;
@@ -109,6 +134,15 @@ int main(int argc, char **argv) {
     CHECK(hipDeviceSynchronize() == hipSuccess);
     CHECK(hipMemcpy(got, out, outer * seg, hipMemcpyDeviceToHost) == hipSuccess);
     for (uint64_t r = 0; r < outer; ++r) CHECK(memcmp(got + r * seg, hsrc + r * pitch + 100, seg) == 0);
+
+    /* the same cut and a whole-row block in one batched call */
+    fstx_slice_desc sd[2] = {{out, src + 100, outer, seg, pitch}, {out + outer * seg, src, 7, pitch, pitch}};
+    CHECK(hipMemset(out, 0, outer * seg + 7 * pitch) == hipSuccess);
+    CHECK(fstx_slice_copy_batch(sd, 2, NULL) == 0);
+    CHECK(hipDeviceSynchronize() == hipSuccess);
+    CHECK(hipMemcpy(got, out, outer * seg + 7 * pitch, hipMemcpyDeviceToHost) == hipSuccess);
+    for (uint64_t r = 0; r < outer; ++r) CHECK(memcmp(got + r * seg, hsrc + r * pitch + 100, seg) == 0);
+    CHECK(memcmp(got + outer * seg, hsrc, 7 * pitch) == 0);
 
     /* two column blocks side by side in one joined matrix, both ways */
     const uint64_t seg2 = 64, joined = seg + seg2;
@@ -124,8 +158,23 @@ int main(int argc, char **argv) {
     fstx_slice2d_desc d2[2] = {{out, src + 100, outer, seg, pitch, joined}, {out + seg, src + 600, outer, seg2, pitch, joined}};
     CHECK(fstx_slice_copy2d_batch(d2, 2, NULL) == 0);
     CHECK(hipDeviceSynchronize() == hipSuccess);
-    CHECK(hipMemcpy(want, out, outer * joined, hipMemcpyDeviceToHost) == hipSuccess);
-    CHECK(memcmp(want, got, outer * joined) == 0); /* `want` is scratch from here on */
+    CHECK(hipMemcpy(tmp, out, outer * joined, hipMemcpyDeviceToHost) == hipSuccess);
+    CHECK(memcmp(tmp, got, outer * joined) == 0);
+
+    /* two joins in one batched call: the same one, and its blocks the other way round */
+    {
+        fstx_join_src swapped[2] = {parts[1], parts[0]};
+        fstx_join_desc jd[2] = {{out, 0, outer, parts, 2, 0}, {out + outer * joined, 0, outer, swapped, 2, 0}};
+        CHECK(hipMemset(out, 0, 2 * outer * joined) == hipSuccess);
+        CHECK(fstx_join_copy_batch(jd, 2, NULL) == 0);
+        CHECK(hipDeviceSynchronize() == hipSuccess);
+        CHECK(hipMemcpy(tmp, out, 2 * outer * joined, hipMemcpyDeviceToHost) == hipSuccess);
+        CHECK(memcmp(tmp, got, outer * joined) == 0);
+        for (uint64_t r = 0; r < outer; ++r) {
+            CHECK(memcmp(tmp + (outer + r) * joined, hsrc + r * pitch + 600, seg2) == 0);
+            CHECK(memcmp(tmp + (outer + r) * joined + seg2, hsrc + r * pitch + 100, seg) == 0);
+        }
+    }
 
     /* fp32 -> bf16 on values of our own */
     enum { NF = 100000 };
@@ -145,6 +194,18 @@ int main(int argc, char **argv) {
     CHECK(hipMemcpy(hb, out, NF * sizeof(uint16_t), hipMemcpyDeviceToHost) == hipSuccess);
     for (int i = 0; i < NF; ++i) CHECK(hb[i] == bf16_of(hf[i]));
 
+    /* the small entry points */
+    CHECK(fstx_get_alignment_size() == 4096);
+    char pci[32];
+    CHECK(fstx_get_device_pci_bus(0, pci, (int)sizeof pci) == 0 && strlen(pci) >= 7 && strchr(pci, ':') != NULL);
+    CHECK(fstx_get_device_pci_bus(0, pci, 2) < 0);
+    void *host = fstx_host_alloc(5000);
+    CHECK(host != NULL && ((uintptr_t)host & 4095) == 0);
+    memset(host, 1, 5000);
+    fstx_host_free(host);
+    fstx_set_debug_log(0);
+    (void)fstx_set_numa_node(0); /* a machine without NUMA information answers with an error; nothing to check but that it returns */
+
     /* error text and argument checks */
     CHECK(strcmp(fstx_strerror(0), "ok") == 0);
     CHECK(fstx_realign_copy_batch(NULL, 3, NULL) == -FSTX_E_INVAL);
@@ -152,6 +213,6 @@ int main(int argc, char **argv) {
 
     hipFree(arena);
     hipFree(out);
-    printf("cabi_check: ok (%llu bytes, 3 read modes, realign, slice, join, convert)\n", (unsigned long long)size);
+    printf("cabi_check: ok (%llu bytes, 3 read modes, shared context, realign, slice, join, convert)\n", (unsigned long long)size);
     return 0;
 }

@@ -173,3 +173,18 @@ def test_the_reference_side_stub_matches_the_header():
     # every library function the stub calls has its signature declared
     called = set(re.findall(r"_lib\.(fstx_\w+)\(", stub))
     assert called <= set(seen), called - set(seen)
+
+
+def test_the_plain_c_program_calls_every_declared_entry_point():
+    """tests/cabi_native/cabi_check.c (run on the GPU by test_loader_gpu) is the C-side user of the
+    header: every function include/fstx.h declares appears in it as a call."""
+    import re
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = open(os.path.join(root, "include", "fstx.h")).read()
+    program = open(os.path.join(root, "tests", "cabi_native", "cabi_check.c")).read()
+    code = re.sub(r"/\*.*?\*/", "", header, flags=re.S)  # comments mention names followed by a bracket
+    declared = set(re.findall(r"\b(fstx_[a-z0-9_]+)\s*\(", code))
+    assert declared == set(_native.EXPORTED_SYMBOLS)
+    missing = sorted(name for name in declared if not re.search(r"\b%s\s*\(" % name, program))
+    assert not missing, missing
