@@ -483,3 +483,44 @@ def test_slice_zero_sized_and_errors(dev):
     with pytest.raises(_native.NativeError):
         _native.slice_copy(a.data_ptr(), a.data_ptr() + 2048, 4, 64, 32, stream())  # pitch < segment
     torch.cuda.synchronize()
+
+
+def test_joins_of_random_geometry_small_and_large(dev):
+    """fstx_join_copy on random jobs against torch's own strided copies, whole destination compared
+    (payload and every byte around it): 1 to 24 sources, segments from 16 bytes to 9 KB, equal and
+    unequal, any alignment of sources and destination, dense and pitched destinations with gaps from
+    one byte to more than the payload, a few rows up to several hundred thousand -- jobs of a few
+    tiles and jobs of many chunks of tiles, common tiles and the tiles at the ends of blocks."""
+    rng = np.random.default_rng(31)
+    lib = _native.lib()
+    for trial in range(60):
+        n = int(rng.choice([1, 1, 2, 3, 5, 7, 14, 24]))
+        hi = int(rng.choice([300, 3000, 9000]))
+        segs = [int(rng.integers(16, hi)) for _ in range(n)]
+        if rng.random() < 0.4:
+            segs = [segs[0]] * n
+        if rng.random() < 0.3:
+            segs = [s // 16 * 16 + 16 for s in segs]
+        budget = 150e6 if trial % 10 == 0 else 8e6
+        rows = int(rng.integers(1, max(2, int(budget // sum(segs)))))
+        rows = min(rows, int(rng.choice([3, 50, 700, 6000, 40000, 300000])))
+        pitches = [s + int(rng.choice([0, 1, 2, 16, 100, 3 * s])) for s in segs]
+        shifts = [int(rng.integers(0, 16)) for _ in range(n)]
+        lead = int(rng.integers(0, 16))
+        gap = int(rng.choice([0, 0, 0, 1, 15, 16, 40, 5000]))
+        row_bytes = sum(segs)
+        dst_pitch = row_bytes + gap
+        srcs = [torch.randint(0, 255, (sh + (rows - 1) * p + s,), dtype=torch.uint8, device=dev)
+                for s, p, sh in zip(segs, pitches, shifts)]
+        dst = torch.full((lead + (rows - 1) * dst_pitch + row_bytes + 64,), 203, dtype=torch.uint8, device=dev)
+        parts = (_native.FstxJoinSrc * n)(*[_native.FstxJoinSrc(t.data_ptr() + sh, s, p)
+                                            for t, sh, s, p in zip(srcs, shifts, segs, pitches)])
+        case = (trial, segs[:4], rows, pitches[:4], gap, lead, shifts[:4])
+        assert lib.fstx_join_copy(dst.data_ptr() + lead, dst_pitch if gap else 0, rows, parts, n, None) == 0, case
+        want = torch.full_like(dst, 203)
+        col = 0
+        for t, sh, s, p in zip(srcs, shifts, segs, pitches):
+            torch.as_strided(want, (rows, s), (dst_pitch, 1), lead + col).copy_(torch.as_strided(t, (rows, s), (p, 1), sh))
+            col += s
+        torch.cuda.synchronize()
+        assert torch.equal(dst, want), case
