@@ -138,8 +138,8 @@ def test_the_product_never_reaches_for_the_oracle_or_scratch_files():
 
 
 def test_the_reference_side_stub_matches_the_header():
-    """INTEGRATION.md shows the ctypes stub a maintainer of the reference would add.  Its code
-    block must parse, and every ``_lib.fstx_*.argtypes`` / ``.restype`` line and the ``_Config``
+    """The integration guide at the repository root shows the ctypes stub a maintainer of the reference
+    would add.  Its code block must parse, and every ``_lib.fstx_*.argtypes`` / ``.restype`` line and the ``_Config``
     fields in it must say what this package's own binding says (which the test above ties to
     ``include/fstx.h``)."""
     import ast
