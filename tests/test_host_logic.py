@@ -9,6 +9,8 @@ regressions (:852-929), the push truth table (test_multi.py:71-82), leak checks.
 """
 from collections import OrderedDict
 
+import os
+
 import pytest
 import torch
 from safetensors.torch import load_file, save_file
@@ -295,3 +297,37 @@ def test_iterate_weights_reports_producer_errors_and_cleans_up(tmp_path):
         PipelineParallel(None, loader_for(None), files, max_concurrent_producers=2)
     with pytest.raises(NotImplementedError):
         PipelineParallel(StubProcessGroup(0, 2), loader_for(StubProcessGroup(0, 2)), files)
+
+
+@pytest.mark.parametrize("queue_size,overlapped", [(0, True), (2, True), (-1, False)])
+def test_the_producer_queues_the_next_batch_before_it_waits_for_this_one(tmp_path, queue_size, overlapped):
+    """With room for a second resident batch the reads of batch k+1 are submitted before batch k is
+    waited for (the transfer then never pauses between batches); with room for one batch only
+    (queue_size -1) every batch is submitted, waited for and consumed before the next begins.
+    Residency never exceeds its bound either way."""
+    from fastsafetensors_amd import PipelineParallel
+
+    files, want = _tiny_files(tmp_path, 5)
+    log = []
+    loader = loader_for(None, log=log)
+    it = PipelineParallel(None, loader, files, queue_size=queue_size)
+    peak = 0
+    n = 0
+    for key, t in it.iterate_weights():
+        peak = max(peak, FW.get_mem_used())
+        assert torch.equal(t, want[key])
+        n += 1
+    it.close()
+    assert n == len(want) and FW.get_mem_used() == 0
+    order = [(what, files.index(path)) for what, path in log]
+    assert [i for what, i in order if what == "submit"] == [0, 1, 2, 3, 4]
+    assert [i for what, i in order if what == "wait"] == [0, 1, 2, 3, 4]
+    at = {entry: pos for pos, entry in enumerate(order)}
+    ahead = [at[("submit", k + 1)] < at[("wait", k)] for k in range(4)]
+    if overlapped:
+        assert any(ahead), order  # (a slow consumer may hold a place now and then; never all the time here)
+    else:
+        assert not any(ahead), order
+    one = max(os.path.getsize(f) for f in files)
+    bound = {0: 2, 2: 3, -1: 1}[queue_size]
+    assert peak <= bound * one
