@@ -189,7 +189,10 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
                          void *dev_base, uint64_t dev_capacity, uint64_t dst_off);
 
 /* Block until every byte of the request is in device memory; returns the byte
- * count or a negative error.  The id is consumed.
+ * count or a negative error.  The id is consumed.  Requests may be waited for in any
+ * order; requests submitted later do not hold the wait up (a caller may queue the next
+ * file's reads before waiting for this one's, and the transfer then runs on without a
+ * pause between the files).
  * nogds_file_reader::wait_read (cpp/ext.cpp:765-776). */
 int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request);
 
