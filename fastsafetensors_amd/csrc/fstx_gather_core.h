@@ -60,12 +60,11 @@ struct alignas(64) Job {
     const char *src;    // nsrc == 1: first byte of the block in row 0
     uint64_t pitch;     // nsrc == 1: bytes between its rows; nsrc > 1: magic_of(equal_seg), or 0
     uint32_t seg;       // nsrc == 1: bytes per row, >= kMinSeg
-    uint32_t flags;     // kByDie, kByRows
+    uint32_t flags;     // kByRows
     uint64_t pitch_magic; // magic_of(dst_pitch); kByRows: magic_of(vectors_per_row(row_bytes))
 };
 
 // Job::flags
-constexpr uint32_t kByDie = 1;  // neighbouring tiles share cache lines (something is not a multiple of 128 bytes)
 constexpr uint32_t kByRows = 2; // vectors are counted row by row (see vectors_per_row)
 
 struct alignas(32) Src {
@@ -81,8 +80,8 @@ constexpr uint32_t kVec = 16;
 constexpr uint32_t kTile = kLanes * kVec; // destination bytes per wavefront
 constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two segments
 
-// Tile order for jobs whose neighbouring tiles share cache lines (a tile = the 1 KiB a wavefront
-// writes; the copy kernels use the same order).  Workgroups reach the eight dies round-robin
+// Tile order of every job (a tile = the 1 KiB a wavefront writes; the copy kernels use the same
+// order).  Workgroups reach the eight dies round-robin
 // (workgroup b runs on die b % 8) and every die has its own L2, so in dispatch order the two
 // tiles either side of a shared line would sit on different dies and the line would be fetched
 // from HBM twice, or a destination line written in two parts.  The tiles are therefore dealt out
@@ -90,8 +89,10 @@ constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two 
 // other, so shared lines are found in that die's L2, while all dies together still sweep one
 // 2 MiB window of the job at a time -- what keeps the memory channels evenly loaded and the dies
 // in step (one contiguous eighth of the job per die measured up to 10 % slower on jobs of
-// 100 MB, and 20 % slower when the eighths alias on the channels).  The last, partial chunk is
-// dealt out in eighths.  A job takes ceil(n_tiles / 8) * 8 workgroups; false = an idle one.
+// 100 MB, and 20 % slower when the eighths alias on the channels).  Jobs in which nothing is
+// shared -- everything on cache-line boundaries -- take the same order: it measured 0-2 % faster
+// than dispatch order on them too.  The last, partial chunk is dealt out in eighths.  A job
+// takes ceil(n_tiles / 8) * 8 workgroups; false = an idle one.
 constexpr uint32_t kDies = 8;
 constexpr uint32_t kRunLog2 = 8;
 FSTX_HD bool tile_for_die(uint32_t lb, uint32_t n_tiles, uint32_t &tile) {
@@ -465,7 +466,7 @@ inline uint64_t rows_per_job(uint64_t dst_pitch, uint64_t row_bytes) {
 // One source: `one` is it and more0 is unused.  Several: they sit at table[more0 .. more0 + nsrc)
 // of the launch and `one` is ignored.
 inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t rows, const Src &one, uint32_t more0,
-                    uint32_t nsrc, uint64_t equal_seg, bool by_die = true) {
+                    uint32_t nsrc, uint64_t equal_seg) {
     const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
     const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
     const bool single = nsrc == 1, by_rows = counts_by_rows(dst_pitch, row_bytes);
@@ -473,7 +474,7 @@ inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t 
     return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,
                (uint32_t)nvec, (uint32_t)(single ? 0 : equal_seg), single ? one.src : nullptr,
                single ? one.pitch : magic_of(equal_seg), single ? one.seg : 0u,
-               (by_die ? kByDie : 0u) | (by_rows ? kByRows : 0u),
+               by_rows ? kByRows : 0u,
                magic_of(by_rows ? vectors_per_row((uint32_t)row_bytes) : dst_pitch)};
 }
 

@@ -188,24 +188,19 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     v4u *dstv = reinterpret_cast<v4u *>(job.dst + head);
     const char *s = job.src + head;
     const uint32_t m = (uint32_t)(uintptr_t)s & (kVecBytes - 1);
-    // Whenever the 1 KiB spans of neighbouring wavefronts share a cache line (source or
-    // destination not on a 128-byte boundary) or a source vector (source shifted), neighbours
-    // run on the same die (tile_for_die).
+    // The 1 KiB spans of neighbouring wavefronts share a cache line (source or destination not
+    // on a 128-byte boundary) or a source vector (source shifted): neighbours run on the same
+    // die, in the tile order of tile_for_die (which also measured faster than dispatch order
+    // when nothing is shared).
     uint32_t tile;
     const bool tile_live = tile_for_die(lb, (uint32_t)((nvec + kBlock - 1) / kBlock), tile);
-    const uint64_t j_by_die = (uint64_t)tile * kBlock + threadIdx.x;
+    const uint64_t j = (uint64_t)tile * kBlock + threadIdx.x;
     if (m == 0) {
-        // source vectors are aligned: a plain streaming copy; in dispatch order when both
-        // sides sit on cache-line boundaries
-        const bool by_die = ((((uintptr_t)s) | (uintptr_t)dstv) & 127) != 0;
-        const uint64_t j = by_die ? j_by_die : (uint64_t)lb * kBlock + threadIdx.x;
+        // source vectors are aligned: a plain streaming copy
         const v4u *srcv = reinterpret_cast<const v4u *>(s);
-        if ((!by_die || tile_live) && j < nvec) {
-            st_stream(ld_stream(srcv + j), dstv + j);
-        }
+        if (tile_live && j < nvec) st_stream(ld_stream(srcv + j), dstv + j);
         return;
     }
-    const uint64_t j = j_by_die;
     const bool live = tile_live && j < nvec; // idle workgroups pad a job to a multiple of eight and to granules
     // Source vectors are loaded at their natural 16-byte alignment; output vector j
     // is bytes [m, m+16) of aligned vectors j and j+1.  Every lane loads vector j
@@ -254,18 +249,10 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     const uint32_t ji = find_job(t, granule_log2, b);
     const SliceJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
-    // in dispatch order when every segment starts on a cache-line boundary on both sides,
-    // else neighbours on the same die (tile_for_die)
-    uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
-#ifndef FSTX_SLICE_NO_REMAP
-    const uint32_t ulog = (uint32_t)(job.pitch_unit >> 56);
-    const uint64_t seg_bytes = (uint64_t)job.seg_units << ulog;
-    if ((((uintptr_t)job.dst | (uintptr_t)job.src | job.pitch_unit | seg_bytes) & 127) != 0) {
-        uint32_t tile;
-        if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
-        u64 = (uint64_t)tile * kBlock + threadIdx.x;
-    }
-#endif
+    // neighbouring workgroups on the same die, in the tile order of tile_for_die
+    uint32_t tile;
+    if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
+    const uint64_t u64 = (uint64_t)tile * kBlock + threadIdx.x;
     if (u64 >= job.total_units) return; // also retires the idle workgroups of a job's last granule
     const uint32_t u = (uint32_t)u64;
     switch ((uint32_t)(job.pitch_unit >> 56)) { // uniform across the workgroup
@@ -303,7 +290,9 @@ __global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t granule_
     const uint32_t ji = find_job(t, granule_log2, b);
     const Slice2dJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
-    const uint64_t u64 = (uint64_t)lb * kBlock + threadIdx.x;
+    uint32_t tile;
+    if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
+    const uint64_t u64 = (uint64_t)tile * kBlock + threadIdx.x;
     if (u64 >= job.total_units) return;
     const uint32_t u = (uint32_t)u64;
     switch (job.unit_log2) { // uniform across the workgroup
@@ -361,11 +350,10 @@ __global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2,
     const fstx_gather::Job job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
     // neighbouring tiles share the cache lines their common border cuts through: neighbours on
-    // the same die (tile_for_die); in dispatch order when everything sits on cache-line
-    // boundaries and nothing is shared
+    // the same die (tile_for_die)
     const uint32_t n_tiles = (job.nvec + fstx_gather::kLanes - 1) / fstx_gather::kLanes;
-    uint32_t tile = lb;
-    if ((job.flags & fstx_gather::kByDie) ? !tile_for_die(lb, n_tiles, tile) : tile >= n_tiles) return; // idle padding of the job's grid
+    uint32_t tile;
+    if (!tile_for_die(lb, n_tiles, tile)) return; // idle padding of the job's grid
     GatherMem<kKeep> mem;
     fstx_gather::gather_lane<kMulti, kPitched>(job, t.more, tile, threadIdx.x, mem);
 }
@@ -517,9 +505,7 @@ __global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t granule_
     const uint32_t ji = find_job(t, granule_log2, b);
     const ConvertJob job = t.fetch(ji);
     uint32_t lb = b - t.first_block[ji];
-    // a job that does not begin on cache lines shares them between neighbouring workgroups:
-    // neighbours on the same die (tile_for_die), as in the copy kernels
-    if ((((uintptr_t)job.src | (uintptr_t)job.dst) & 127) != 0) {
+    { // neighbouring workgroups on the same die, in the tile order of tile_for_die, as in the copy kernels
         const uint32_t per_block_log2 = 7 + (job.src_type < 2 ? job.src_type : 2); // 64 lanes x 16 bytes of f64 / f32 / 16-bit
         const uint32_t n_tiles = (uint32_t)((job.n_elems + (1ull << per_block_log2) - 1) >> per_block_log2);
         uint32_t tile;
@@ -625,7 +611,7 @@ struct GatherBatch {
     int add(void *dst, uint64_t dst_pitch, uint64_t rows, const fstx_join_src *srcs, uint32_t n) {
         fstx_join_src live[kGatherMore];
         uint32_t m = 0;
-        uint64_t row_bytes = 0, equal = 0, min_seg = ~0ull, bits = (uint64_t)(uintptr_t)dst;
+        uint64_t row_bytes = 0, equal = 0, min_seg = ~0ull;
         for (uint32_t i = 0; i < n; ++i) {
             if (srcs[i].seg_bytes == 0) continue;
             if (m == 0) equal = srcs[i].seg_bytes;
@@ -633,10 +619,8 @@ struct GatherBatch {
             if (srcs[i].seg_bytes < min_seg) min_seg = srcs[i].seg_bytes;
             live[m++] = srcs[i];
             row_bytes += srcs[i].seg_bytes;
-            bits |= (uint64_t)(uintptr_t)srcs[i].src | srcs[i].seg_bytes | srcs[i].src_pitch;
         }
         if (dst_pitch == 0) dst_pitch = row_bytes;
-        const bool lines_shared = ((bits | dst_pitch) & 127) != 0;
         // rows per job: 32-bit positions, and no more tiles than one job may take
         uint64_t per_job = fstx_gather::rows_per_job(dst_pitch, row_bytes);
         const uint64_t by_tiles = lim.job * fstx_gather::kTile / dst_pitch;
@@ -649,7 +633,7 @@ struct GatherBatch {
                                         (uint32_t)live[i].seg_bytes, (uint32_t)col, 0};
             };
             fstx_gather::Job job = fstx_gather::make_job(static_cast<char *>(dst) + row * dst_pitch, dst_pitch, row_bytes,
-                                                         part, source(0, 0), 0, m, m > 1 ? equal : 0, lines_shared);
+                                                         part, source(0, 0), 0, m, m > 1 ? equal : 0);
             const uint64_t need = (fstx_gather::tiles_of(job) + kXcds - 1) / kXcds * kXcds; // whole eighths
             if (nj == kGatherJobs || (m > 1 && ns + m > kGatherMore) || tiles + need > lim.launch) {
                 int rc = flush();
@@ -860,14 +844,14 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         for (uint64_t row = 0; row < d.outer; row += rows_per_job) {
             const uint64_t rows = d.outer - row < rows_per_job ? d.outer - row : rows_per_job;
             const uint64_t units = rows * seg_units;
-            if (k == kJobs || blocks + blocks_for(units) > lim.launch) {
+            if (k == kJobs || blocks + blocks_for(units) + kXcds > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
             t.job[k] = Slice2dJob{static_cast<char *>(d.dst) + row * d.dst_pitch,
                                   static_cast<const char *>(d.src) + row * d.src_pitch,
                                   d.src_pitch, d.dst_pitch, (uint32_t)seg_units, (uint32_t)units, ul, 0, 0, 0};
-            blocks_of[k] = blocks_for(units);
+            blocks_of[k] = (blocks_for(units) + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
             blocks += blocks_of[k];
             ++k;
         }
@@ -967,9 +951,7 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         const uint64_t piece = lim.job * per_block; // elements one job may take
         for (uint64_t done = 0; done < d.n_elems; done += piece) {
             const uint64_t len = d.n_elems - done < piece ? d.n_elems - done : piece;
-            uint64_t need = (len + per_block - 1) / per_block;
-            if ((((uintptr_t)(db + done * ds) | (uintptr_t)(sb + done * ss)) & 127) != 0)
-                need = (need + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
+            const uint64_t need = ((len + per_block - 1) / per_block + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
             if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
