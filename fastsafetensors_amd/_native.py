@@ -18,11 +18,13 @@ _LIB_NAME = "libfstx.so"
 _lib: Optional[ctypes.CDLL] = None
 _lib_lock = threading.Lock()
 
-FSTX_ABI_VERSION = 2
+FSTX_ABI_VERSION = 3
 FSTX_BATCH_MAX = 48
 READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
 ADAPTIVE_DEPTH = 1
 PROBE_NO_COPY, PROBE_NO_READ = 2, 4
+NO_PRETOUCH = 8
+STORAGE_KNOWN, STORAGE_ROTATIONAL, STORAGE_VIRTIO = 1, 2, 4
 READ_MODES = {"auto": READ_AUTO, "buffered": READ_BUFFERED, "direct": READ_DIRECT}
 
 
@@ -50,10 +52,14 @@ class FstxConfig(ctypes.Structure):
     ]
 
 
+_METRICS_SIGNED = ("numa_node", "ring_node", "first_bind_error")
+
+
 class FstxMetrics(ctypes.Structure):
     _fields_ = [
-        (name, ctypes.c_uint64)
+        (name, ctypes.c_int64 if name in _METRICS_SIGNED else ctypes.c_uint64)
         for name in (
+            "struct_size",
             "bounce_buffer_bytes",
             "bytes_read",
             "bytes_copied",
@@ -66,8 +72,25 @@ class FstxMetrics(ctypes.Structure):
             "direct_depth",
             "direct_reads",
             "create_ns",
+            "numa_node",
+            "workers_on_node",
+            "ring_node",
+            "bind_errors",
+            "first_bind_error",
+            "pretouched_bytes",
+            "direct_read_bytes",
+            "direct_steered",
+            "staging_buffers_max",
+            "storage_nr_requests",
+            "storage_max_sectors_kb",
+            "storage_flags",
         )
     ]
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        if not self.struct_size:
+            self.struct_size = ctypes.sizeof(FstxMetrics)
 
 
 class FstxCopyDesc(ctypes.Structure):
@@ -139,6 +162,7 @@ _SIGNATURES = {
     "fstx_get_alignment_size": (ctypes.c_int, []),
     "fstx_get_device_pci_bus": (ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, ctypes.c_int]),
     "fstx_set_numa_node": (ctypes.c_int, [ctypes.c_int]),
+    "fstx_node_cpus": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.c_int]),
     "fstx_set_debug_log": (None, [ctypes.c_int]),
     "fstx_bounce_buffer_bytes": (ctypes.c_uint64, []),
     "fstx_strerror": (ctypes.c_char_p, [ctypes.c_int64]),
@@ -252,6 +276,13 @@ def get_device_pci_bus(device_id: int) -> str:
 
 def set_numa_node(node: int) -> int:
     return 0 if lib().fstx_set_numa_node(int(node)) >= 0 else -1
+
+
+def node_cpus(node: int) -> List[int]:
+    """CPUs of a NUMA node as the library reads them from sysfs; empty when the node is unknown."""
+    buf = (ctypes.c_int * 4096)()
+    n = lib().fstx_node_cpus(int(node), buf, len(buf))
+    return list(buf[: min(n, len(buf))]) if n > 0 else []
 
 
 def bounce_buffer_bytes() -> int:

@@ -47,8 +47,10 @@
 #include <errno.h>
 #include <fcntl.h>
 #include <sched.h>
+#include <limits.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
+#include <sys/sysmacros.h>
 #include <sys/syscall.h>
 #include <unistd.h>
 
@@ -73,36 +75,64 @@ std::atomic<int> g_debug{0};
 std::atomic<int64_t> g_bounce_bytes{0};
 std::atomic<uint32_t> g_depth_hint{2}; // O_DIRECT depth the last adaptive context settled on
 
-// ---- NUMA ------------------------------------------------------------------
+// ---- NUMA and storage facts from sysfs --------------------------------------------
 
-// CPUs of a node from sysfs ("0-15,32-47"); empty when unknown
-std::vector<int> node_cpus(int node) {
-    std::vector<int> cpus;
-    char path[96];
-    std::snprintf(path, sizeof path, "/sys/devices/system/node/node%d/cpulist", node);
-    FILE *f = std::fopen(path, "r");
-    if (!f) return cpus;
+// "/sys" unless FSTX_SYSFS_ROOT names another tree (tests lay one out with the nodes and
+// block devices they want the library to see)
+std::string sysfs_root() {
+    const char *e = std::getenv("FSTX_SYSFS_ROOT");
+    return e && *e ? std::string(e) : std::string("/sys");
+}
+
+// first line of a sysfs attribute, without the newline; false when unreadable
+bool read_sysfs_line(const std::string &path, std::string &out) {
+    FILE *f = std::fopen(path.c_str(), "r");
+    if (!f) return false;
     char buf[4096];
-    if (std::fgets(buf, sizeof buf, f)) {
-        char *p = buf;
-        while (*p && *p != '\n') {
-            char *end;
-            long a = std::strtol(p, &end, 10);
-            if (end == p) break;
-            long b = a;
-            p = end;
-            if (*p == '-') {
-                b = std::strtol(p + 1, &end, 10);
-                p = end;
-            }
-            for (long c = a; c <= b && c < CPU_SETSIZE; ++c) cpus.push_back((int)c);
-            if (*p == ',') ++p;
-        }
-    }
+    const bool ok = std::fgets(buf, sizeof buf, f) != nullptr;
     std::fclose(f);
+    if (!ok) return false;
+    out.assign(buf);
+    while (!out.empty() && (out.back() == '\n' || out.back() == ' ')) out.pop_back();
+    return true;
+}
+
+// "0-3,8,10-11" -> 0 1 2 3 8 10 11 (the kernel's cpulist format); stops at the first thing it
+// cannot read and returns what it had
+std::vector<int> parse_cpulist(const char *text) {
+    std::vector<int> cpus;
+    const char *p = text;
+    while (*p && *p != '\n') {
+        char *end;
+        long a = std::strtol(p, &end, 10);
+        if (end == p || a < 0) break;
+        long b = a;
+        p = end;
+        if (*p == '-') {
+            b = std::strtol(p + 1, &end, 10);
+            if (end == p + 1) break;
+            p = end;
+        }
+        for (long c = a; c <= b && c < CPU_SETSIZE; ++c) cpus.push_back((int)c);
+        if (*p == ',') ++p;
+        else break;
+    }
     return cpus;
 }
 
+// CPUs of a node; empty when the node is unknown
+std::vector<int> node_cpus(int node) {
+    std::string line;
+    if (node < 0 || !read_sysfs_line(sysfs_root() + "/devices/system/node/node" + std::to_string(node) + "/cpulist", line))
+        return {};
+    return parse_cpulist(line.c_str());
+}
+
+constexpr int kMaxNode = 1024;
+
+// Restrict the calling thread to the node's CPUs and prefer the node's memory
+// (MPOL_PREFERRED: allocate there while it has room).  0, or the first failure as -errno;
+// -ENODEV for a node without CPUs.
 int bind_thread_to_node(int node) {
     if (node < 0) return 0;
     std::vector<int> cpus = node_cpus(node);
@@ -111,14 +141,89 @@ int bind_thread_to_node(int node) {
     CPU_ZERO(&set);
     for (int c : cpus) CPU_SET(c, &set);
     if (sched_setaffinity(0, sizeof set, &set) != 0) return -errno;
+    if (node >= kMaxNode) return -EINVAL;
 #ifdef SYS_set_mempolicy
-    if (node < 64) {
-        // MPOL_PREFERRED = 1: allocate on this node while it has room
-        unsigned long mask = 1ul << node;
-        (void)syscall(SYS_set_mempolicy, 1, &mask, sizeof(mask) * 8);
-    }
+    unsigned long mask[kMaxNode / (8 * sizeof(unsigned long))] = {0};
+    mask[node / (8 * sizeof(unsigned long))] = 1ul << (node % (8 * sizeof(unsigned long)));
+    if (syscall(SYS_set_mempolicy, 1 /* MPOL_PREFERRED */, mask, (unsigned long)kMaxNode + 1) != 0) return -errno;
 #endif
     return 0;
+}
+
+// whether the calling thread may run on CPUs of `node` only (and on at least one of them)
+bool thread_sits_on_node(int node) {
+    std::vector<int> cpus = node_cpus(node);
+    cpu_set_t have;
+    CPU_ZERO(&have);
+    if (cpus.empty() || sched_getaffinity(0, sizeof have, &have) != 0 || CPU_COUNT(&have) == 0) return false;
+    cpu_set_t of_node;
+    CPU_ZERO(&of_node);
+    for (int c : cpus) CPU_SET(c, &of_node);
+    for (int c = 0; c < CPU_SETSIZE; ++c)
+        if (CPU_ISSET(c, &have) && !CPU_ISSET(c, &of_node)) return false;
+    return true;
+}
+
+// node that holds the page at `addr` (which must have been touched), or -1 when the kernel
+// does not say (memory that is mapped from a device driver has no struct page to ask about)
+int node_of_address(const void *addr) {
+#ifdef SYS_get_mempolicy
+    int node = -1;
+    if (syscall(SYS_get_mempolicy, &node, nullptr, 0ul, addr, 3ul /* MPOL_F_NODE | MPOL_F_ADDR */) == 0) return node;
+#endif
+#ifdef SYS_move_pages
+    void *pages[1] = {const_cast<void *>(addr)};
+    int status[1] = {-1};
+    if (syscall(SYS_move_pages, 0, 1ul, pages, nullptr, status, 0) == 0 && status[0] >= 0) return status[0];
+#endif
+    return -1;
+}
+
+// What the block layer says about the device under a file: how many requests its queue
+// holds, how large one request may be, whether it seeks, whether it is a paravirtual disk.
+struct StorageFacts {
+    bool known = false;
+    uint64_t nr_requests = 0, max_sectors_kb = 0;
+    bool rotational = false, virtio = false;
+    std::string name;
+};
+
+StorageFacts storage_facts(dev_t dev) {
+    StorageFacts out;
+    const std::string base = sysfs_root() + "/dev/block/" + std::to_string(major(dev)) + ":" + std::to_string(minor(dev));
+    // a partition has no queue of its own: its parent directory is the whole device
+    std::string dir = base, line;
+    if (!read_sysfs_line(dir + "/queue/nr_requests", line)) {
+        dir = base + "/..";
+        if (!read_sysfs_line(dir + "/queue/nr_requests", line)) return out;
+    }
+    out.nr_requests = std::strtoull(line.c_str(), nullptr, 10);
+    if (read_sysfs_line(dir + "/queue/max_sectors_kb", line)) out.max_sectors_kb = std::strtoull(line.c_str(), nullptr, 10);
+    if (read_sysfs_line(dir + "/queue/rotational", line)) out.rotational = line == "1";
+    char resolved[PATH_MAX];
+    if (realpath(dir.c_str(), resolved)) {
+        out.name = resolved;
+        const size_t cut = out.name.rfind('/');
+        if (cut != std::string::npos) out.name = out.name.substr(cut + 1);
+        // virtio-blk disks are named vdX and hang off a virtioN device
+        out.virtio = out.name.rfind("vd", 0) == 0 || std::strstr(resolved, "/virtio") != nullptr;
+    }
+    out.known = out.nr_requests > 0 && out.max_sectors_kb > 0;
+    return out;
+}
+
+// MemAvailable of /proc/meminfo (of $FSTX_PROCFS_ROOT/meminfo in tests); 0 when unknown
+uint64_t mem_available_bytes() {
+    const char *e = std::getenv("FSTX_PROCFS_ROOT");
+    const std::string path = std::string(e && *e ? e : "/proc") + "/meminfo";
+    FILE *f = std::fopen(path.c_str(), "r");
+    if (!f) return 0;
+    char line[256];
+    uint64_t kb = 0;
+    while (std::fgets(line, sizeof line, f))
+        if (std::sscanf(line, "MemAvailable: %llu kB", (unsigned long long *)&kb) == 1) break;
+    std::fclose(f);
+    return kb * 1024;
 }
 
 // ---- data model ------------------------------------------------------------
@@ -173,14 +278,25 @@ struct Slot {
 };
 
 // Bounds the O_DIRECT preads in flight.  Storage differs a lot in the queue depth
-// it wants (a virtio disk peaks at 2, an NVMe array at 32 or more); with
-// FSTX_ADAPTIVE_DEPTH the depth is steered while reading: every window of
-// completed blocks yields a rate; a step that raised the rate is repeated, a
-// step that lowered it is undone, and a change within the noise leaves the depth alone.
+// it wants (a virtio disk peaks at 1 or 2, an NVMe array at 16 or more); a steered gate
+// finds it while reading.  Completed reads are counted in windows; a window yields a rate.
+// From a measured base the gate tries one read more: a gain of 8 % keeps the step and tries
+// the next one, anything less takes it back.  Then it tries one read fewer, and keeps that
+// when the rate holds (within 3 %): of two depths that read equally fast the smaller one
+// needs fewer staging buffers and keeps the requests in order.  After a step in each
+// direction has failed the depth rests for a few windows before the next round.
 class Gate {
   public:
-    Gate(uint32_t start, uint32_t hi, bool adaptive)
-        : limit_(std::max(1u, std::min(start, hi))), hi_(std::max(1u, hi)), adaptive_(adaptive) {}
+    Gate(uint32_t start, uint32_t hi, bool adaptive) { configure(start, hi, adaptive); }
+    // (re)set depth, ceiling and steering; reads in flight keep their tokens
+    void configure(uint32_t start, uint32_t hi, bool adaptive) {
+        std::lock_guard<std::mutex> lk(m_);
+        hi_ = std::max(1u, hi);
+        limit_ = std::max(1u, std::min(start, hi_));
+        adaptive_ = adaptive;
+        phase_ = kBase;
+        win_blocks_ = 0;
+    }
     // take a token if one is free; callers that must start their reads in file
     // order call this while they hold the block queue's lock
     bool try_enter() {
@@ -198,45 +314,94 @@ class Gate {
         std::lock_guard<std::mutex> lk(m_);
         return limit_;
     }
-
-  private:
-    void steer(uint64_t bytes) {
-        const uint64_t now = now_ns();
-        if (win_blocks_ == 0 || now - last_done_ > 50'000'000ull) { // first block, or reading paused
-            win_t0_ = now;
-            win_bytes_ = 0;
-            win_blocks_ = 0;
-            if (now - last_done_ > 50'000'000ull) last_rate_ = 0;
-        }
-        last_done_ = now;
-        win_bytes_ += bytes;
-        if (++win_blocks_ < std::max(16u, 6 * limit_) || now == win_t0_) return;
-        const double rate = (double)win_bytes_ / (double)(now - win_t0_);
-        int step = dir_;
-        if (last_rate_ > 0) {
-            if (rate < 0.92 * last_rate_) step = dir_ = -dir_;   // that step hurt: go back
-            else if (rate < 1.08 * last_rate_) step = 0;         // within the noise: stay
-        }
-        last_rate_ = rate;
-        int64_t next = (int64_t)limit_ + step;
-        if (next < 1) { next = 1; dir_ = 1; }
-        if (next > (int64_t)hi_) { next = hi_; dir_ = -1; }
-        limit_ = (uint32_t)next;
-        win_blocks_ = 0;
+    // the depth that was last found good: a step that is still being tried does not count
+    uint32_t settled() {
+        std::lock_guard<std::mutex> lk(m_);
+        if (phase_ == kTryUp && limit_ > 1) return limit_ - 1;
+        if (phase_ == kTryDown && limit_ < hi_) return limit_ + 1;
+        return limit_;
     }
 
+  private:
+    enum Phase { kBase, kTryUp, kTryDown, kRest };
+
+    void steer(uint64_t bytes) {
+        const uint64_t now = now_ns();
+        const bool paused = last_done_ != 0 && now - last_done_ > 50'000'000ull;
+        last_done_ = now;
+        if (paused) { // what was measured before the pause is stale: take a trial step back, start over
+            if (phase_ == kTryUp && limit_ > 1) --limit_;
+            if (phase_ == kTryDown && limit_ < hi_) ++limit_;
+            phase_ = kBase;
+            went_up_ = false;
+            win_blocks_ = 0;
+        }
+        if (win_blocks_ == 0) { // this read opens a window: its own bytes came before the clock started
+            win_t0_ = now;
+            win_bytes_ = 0;
+            win_blocks_ = 1;
+            return;
+        }
+        win_bytes_ += bytes;
+        // a window: at least 8 reads, four per read in flight, and 20 ms (short windows of small reads measure the scheduler)
+        if (++win_blocks_ <= std::max(8u, 4 * limit_) || now - win_t0_ < 20'000'000ull) return;
+        const double rate = (double)win_bytes_ / (double)(now - win_t0_);
+        win_blocks_ = 0;
+        fstx_internal::debug("gate: depth %u phase %d rate %.3f GB/s base %.3f", limit_, (int)phase_, rate, base_rate_);
+        auto rest = [&] { phase_ = kRest, rest_ = kRestWindows; };
+        switch (phase_) {
+        case kBase:
+            base_rate_ = rate;
+            went_up_ = false;
+            if (limit_ < hi_) ++limit_, phase_ = kTryUp;
+            else if (limit_ > 1) --limit_, phase_ = kTryDown;
+            break;
+        case kTryUp:
+            if (rate >= 1.08 * base_rate_) { // worth it: keep the step and try the next one
+                base_rate_ = rate;
+                went_up_ = true;
+                if (limit_ < hi_) ++limit_;
+                else rest();
+            } else {
+                --limit_;
+                // a round that gained nothing upwards looks downwards next
+                if (!went_up_ && limit_ > 1) --limit_, phase_ = kTryDown;
+                else rest();
+            }
+            break;
+        case kTryDown:
+            if (rate >= 0.97 * base_rate_) { // no worse with one read fewer: keep
+                base_rate_ = std::max(base_rate_, rate);
+                if (limit_ > 1) --limit_;
+                else rest();
+            } else {
+                ++limit_;
+                rest();
+            }
+            break;
+        case kRest:
+            if (--rest_ == 0) phase_ = kBase;
+            break;
+        }
+    }
+
+    static constexpr uint32_t kRestWindows = 6;
     std::mutex m_;
-    uint32_t limit_, hi_, busy_ = 0;
-    bool adaptive_;
-    int dir_ = 1;
-    double last_rate_ = 0;
+    uint32_t limit_ = 1, hi_ = 1, busy_ = 0;
+    bool adaptive_ = false;
+    Phase phase_ = kBase;
+    bool went_up_ = false; // the last round of upward steps kept at least one: no downward try after it
+    uint32_t rest_ = 0;
+    double base_rate_ = 0;
     uint64_t win_t0_ = 0, win_bytes_ = 0, last_done_ = 0;
     uint32_t win_blocks_ = 0;
 };
 
 struct Counters {
     std::atomic<uint64_t> bytes_read{0}, bytes_copied{0}, blocks_buffered{0}, blocks_direct{0},
-        read_ns{0}, stage_ns{0}, slot_wait_ns{0}, direct_fallbacks{0}, direct_reads{0};
+        read_ns{0}, stage_ns{0}, slot_wait_ns{0}, direct_fallbacks{0}, direct_reads{0}, workers_on_node{0},
+        bind_errors{0}, pretouched_bytes{0};
+    std::atomic<int64_t> first_bind_error{0};
 };
 
 } // namespace
@@ -261,7 +426,9 @@ struct fstx_ctx {
     uint64_t queue_pops = 0;               // blocks taken off `queue` so far (q_mutex)
     uint64_t head_verdict_for = ~0ull;     // value of queue_pops the cached verdict belongs to
     bool head_wants_direct = false;        // whether the block at the head of `queue` is to be read with O_DIRECT
+    bool extending = false;                // a worker asks the page cache how far its run may reach: `queue` is its alone meanwhile
     bool closing = false;
+    std::atomic<bool> work_seen{false};    // something was queued at least once: the workers stop touching their idle slots
 
     std::mutex done_mutex;
     std::condition_variable done_cv;
@@ -286,6 +453,11 @@ struct fstx_ctx {
     int64_t next_request = 1;
 
     Counters ctr;
+    // Shape of the O_DIRECT reads: what the configuration fixes, and for what it leaves at 0 the
+    // figures of the block device under the first file that is opened for O_DIRECT (q_mutex)
+    bool shape_settled = false;
+    StorageFacts storage;
+    int ring_node = -1;        // node of the ring's first page, where the kernel says (ready_mutex)
     uint64_t direct_bytes = 0; // bytes one O_DIRECT pread may cover
     // ordinary page-backed blocks that O_DIRECT reads land in; handed out together
     // with the read token (under q_mutex), returned after the last byte left for the ring
@@ -306,6 +478,12 @@ StageLoan::~StageLoan() {
 }
 
 // ---- reading one block -------------------------------------------------------
+
+} // namespace
+// Test seam: a host-only test build may define this to put a storage model (latency, bandwidth,
+// parallelism) behind every O_DIRECT read; the shipped library leaves it undefined.
+extern "C" __attribute__((weak)) void fstx_test_after_direct_read(uint64_t bytes);
+namespace {
 
 // pread until `want` bytes arrived, EOF or error; returns bytes or -errno
 int64_t pread_full(int fd, char *buf, uint64_t want, uint64_t off) {
@@ -484,6 +662,7 @@ struct Worker {
         uint64_t t0 = now_ns();
         int64_t got = ctx->no_read ? (int64_t)std::min(want, align_up(f.size, kPage) - window)
                                    : pread_full(f.fd_direct, stage, want, window);
+        if (fstx_test_after_direct_read && got > 0) fstx_test_after_direct_read((uint64_t)got);
         uint64_t t1 = now_ns();
         ctx->ctr.direct_reads.fetch_add(1, std::memory_order_relaxed);
         release_token(got > 0 ? (uint64_t)got : 0);
@@ -595,8 +774,37 @@ struct Worker {
         return 0;
     }
 
+    // Map the pages of this worker's idle slots into the process before the first block needs
+    // them: pinned memory is mapped page by page at its first touch, and that costs more per
+    // byte than copying it to the device (measured 0.34 ms per MiB on one thread, 0.06 with
+    // sixteen).  Runs while the creating thread still builds the rest of the context and its
+    // caller parses file headers, and stops for good as soon as anything is queued -- from
+    // then on the reads touch what is left as they go, and a slot may hold data.
+    void pretouch() {
+        uint64_t done = 0;
+        for (Slot &slot : *mine)
+            for (uint64_t at = 0; at < ctx->slot_bytes; at += kPage) {
+                if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
+                    ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
+                    return;
+                }
+                *(volatile char *)(slot.host + at) = 0;
+                done += kPage;
+            }
+        ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
+    }
+
     void run() {
-        bind_thread_to_node(ctx->cfg.numa_node);
+        const int node = ctx->cfg.numa_node;
+        if (node >= 0) {
+            const int bound = bind_thread_to_node(node);
+            if (bound < 0) {
+                ctx->ctr.bind_errors.fetch_add(1, std::memory_order_relaxed);
+                int64_t none = 0;
+                ctx->ctr.first_bind_error.compare_exchange_strong(none, bound);
+            }
+            if (thread_sits_on_node(node)) ctx->ctr.workers_on_node.fetch_add(1, std::memory_order_relaxed);
+        }
         int64_t dev_rc = fstx_dev::set_device(ctx->cfg.device_id);
         mine = &ctx->slots[index];
         if (dev_rc == 0) dev_rc = make_slots();
@@ -608,13 +816,14 @@ struct Worker {
         ctx->ready_cv.notify_all();
         stream_ix = index % (uint32_t)ctx->streams.size();
         stream = ctx->streams[stream_ix];
+        if (dev_rc == 0 && !ctx->no_read && !(ctx->cfg.flags & FSTX_NO_PRETOUCH)) pretouch();
         std::vector<Block> run;
         std::vector<int64_t> status;
         for (;;) {
             run.clear();
             bool direct = false;
             Staged todo;
-            bool have_staged = false;
+            bool have_staged = false, woke_others = false;
             {
                 // Blocks leave the queue in file order.  A block that needs O_DIRECT is
                 // taken together with its token, under this lock, so that the reads reach
@@ -628,8 +837,11 @@ struct Worker {
                     have_staged = true;
                 };
                 for (;;) {
-                    ctx->q_cv.wait(lk, [&] { return ctx->closing || !ctx->queue.empty() || !ctx->staged.empty(); });
-                    if (ctx->queue.empty()) {
+                    // (while another worker extends its run, the queue is that worker's alone)
+                    ctx->q_cv.wait(lk, [&] {
+                        return !ctx->staged.empty() || (!ctx->extending && (ctx->closing || !ctx->queue.empty()));
+                    });
+                    if (ctx->extending || ctx->queue.empty()) {
                         if (!ctx->staged.empty()) take_staged();
                         break; // with nothing taken: closing and drained
                     }
@@ -670,12 +882,22 @@ struct Worker {
                     pop();
                     if (direct) {
                         // extend the run with the blocks that follow it in the file; in AUTO mode
-                        // only as far as the file is not in the page cache (one mincore call over
-                        // the stretch the run may cover)
+                        // only as far as the file is not in the page cache.  That is one mincore
+                        // call over the stretch the run may cover (262,144 pages for 1 GiB), made
+                        // with the lock released: `extending` keeps the queue for this worker
+                        // while the others go on shipping staged blocks.
                         ++ctx->burst_runs;
                         FileEntry &f = *run[0].req->file;
                         Residency seen;
-                        if (f.mode == FSTX_READ_AUTO) seen.probe(f, run[0].file_off + run[0].len, run[0].file_off + limit);
+                        if (f.mode == FSTX_READ_AUTO && !ctx->queue.empty()) {
+                            const uint64_t from = run[0].file_off + run[0].len, to = run[0].file_off + limit;
+                            ctx->extending = true;
+                            lk.unlock();
+                            seen.probe(f, from, to);
+                            lk.lock();
+                            ctx->extending = false;
+                            woke_others = true;
+                        }
                         uint64_t bytes = run[0].len + run[0].file_off % kPage;
                         while (!ctx->queue.empty()) {
                             const Block &nx = ctx->queue.front();
@@ -690,6 +912,7 @@ struct Worker {
                     if (ctx->queue.empty()) ctx->burst_runs = 0; // the next read starts a new burst
                 }
             }
+            if (woke_others) ctx->q_cv.notify_all(); // the queue is everybody's again
             if (have_staged) {
                 ship_staged(todo);
                 continue;
@@ -762,9 +985,14 @@ int fstx_get_device_pci_bus(int device_id, char *out, int len) {
     return fstx_dev::pci_bus_id(device_id, out, len);
 }
 
-int fstx_set_numa_node(int numa_node) {
-    int rc = bind_thread_to_node(numa_node);
-    return rc < 0 ? rc : 0;
+int fstx_set_numa_node(int numa_node) { return bind_thread_to_node(numa_node); }
+
+int fstx_node_cpus(int numa_node, int *cpus, int capacity) {
+    if (numa_node < 0 || capacity < 0 || (capacity && !cpus)) return -FSTX_E_INVAL;
+    const std::vector<int> found = node_cpus(numa_node);
+    if (found.empty()) return -ENODEV;
+    for (size_t i = 0; i < found.size() && i < (size_t)capacity; ++i) cpus[i] = found[i];
+    return (int)found.size();
 }
 
 void *fstx_host_alloc(uint64_t length) {
@@ -802,13 +1030,13 @@ int normalize(fstx_config &cfg) {
     if (cfg.n_streams == 0) cfg.n_streams = 4;
     if (cfg.block_bytes == 0) cfg.block_bytes = kDefaultBlock;
     if (cfg.slots_per_thread == 0) cfg.slots_per_thread = 2;
-    const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
-    if (cfg.max_direct_reads == 0) cfg.max_direct_reads = adaptive_depth ? g_depth_hint.load() : 1;
-    if (cfg.direct_read_bytes == 0) cfg.direct_read_bytes = 1ull << 30;
+    // max_direct_reads and direct_read_bytes stay 0 when the caller leaves them open: they are
+    // settled from the block device under the first file that is opened for O_DIRECT
     if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 || cfg.slots_per_thread > 64 ||
-        (cfg.flags & ~(FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_NO_COPY | FSTX_PROBE_NO_READ)))
+        (cfg.flags & ~(FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_NO_COPY | FSTX_PROBE_NO_READ | FSTX_NO_PRETOUCH)))
         return -FSTX_E_INVAL;
-    cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
+    if (cfg.direct_read_bytes)
+        cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
     if (cfg.direct_ramp_kb == 0) cfg.direct_ramp_kb = 64 * 1024;
     cfg.n_streams = std::min(cfg.n_streams, cfg.n_threads);
     cfg.struct_size = sizeof(fstx_config);
@@ -858,6 +1086,51 @@ bool same_config(const fstx_config &a, const fstx_config &b) {
            a.direct_ramp_kb == b.direct_ramp_kb;
 }
 
+// Depth and size of the O_DIRECT reads (call with q_mutex held, or before the workers exist).
+// What the configuration names is kept.  What it leaves at 0 follows the device: one request
+// queue's worth of bytes (nr_requests x max_sectors_kb, between 64 MiB and 1 GiB) is the budget.
+//   * a paravirtual or rotating disk, or one the block layer tells nothing about, is read with
+//     ONE request in flight that carries the whole budget (measured on a virtio disk: two
+//     readers, or the same bytes in smaller requests, lose up to half the rate);
+//   * anything else (NVMe, SCSI SSDs, md / dm arrays of them) wants several requests in flight:
+//     reads of a quarter of the budget, depth 2 to begin with, steered while reading.
+// The staging buffers those reads land in are ordinary memory: their number times their size
+// stays under 1/16 of MemAvailable (at least 128 MiB).
+void settle_direct_shape(fstx_ctx *ctx, const StorageFacts &facts) {
+    const fstx_config &cfg = ctx->cfg;
+    const bool asked_adaptive = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
+    uint64_t budget = 1ull << 30;
+    if (facts.known) budget = std::min<uint64_t>(1ull << 30, std::max<uint64_t>(64ull << 20, facts.nr_requests * facts.max_sectors_kb * 1024));
+    const bool serial = !facts.known || facts.virtio || facts.rotational;
+    const bool adaptive = asked_adaptive || (cfg.max_direct_reads == 0 && !serial);
+    uint32_t depth = cfg.max_direct_reads;
+    if (depth == 0) depth = adaptive ? g_depth_hint.load() : 1; // the hint: where the last steered context ended, 2 at first
+    const uint32_t hi = std::min(cfg.n_threads, 32u);
+    uint64_t bytes = cfg.direct_read_bytes;
+    if (bytes == 0) bytes = adaptive ? std::max<uint64_t>(64ull << 20, budget / 4) : budget;
+    bytes = std::max(cfg.block_bytes, align_down(bytes, cfg.block_bytes));
+    // one staging buffer per read in flight plus one that is being emptied into the ring meanwhile
+    uint32_t stages = (adaptive ? std::min(hi, 16u) : std::min(depth, cfg.n_threads)) + 1;
+    if (cfg.direct_read_bytes == 0) {
+        const uint64_t avail = mem_available_bytes();
+        const uint64_t cap = std::max<uint64_t>(128ull << 20, (avail ? avail : (64ull << 30)) / 16);
+        const uint32_t fewest = adaptive ? 3 : 2;
+        while (stages > fewest && stages * bytes > cap) --stages;
+        if (stages * bytes > cap) bytes = std::max(cfg.block_bytes, align_down(cap / stages, cfg.block_bytes));
+    }
+    ctx->storage = facts;
+    ctx->direct_bytes = bytes;
+    ctx->ramp_bytes = std::max(cfg.block_bytes, align_down((uint64_t)cfg.direct_ramp_kb * 1024, cfg.block_bytes));
+    ctx->stage_max = stages;
+    ctx->adaptive_depth = adaptive;
+    ctx->direct_gate->configure(depth, hi, adaptive);
+    ctx->shape_settled = true;
+    fstx_internal::debug("direct reads: device %s (nr_requests %llu, max_sectors_kb %llu%s%s) -> %llu bytes per read, depth %u%s, %u staging buffers",
+                         facts.known ? facts.name.c_str() : "unknown", (unsigned long long)facts.nr_requests,
+                         (unsigned long long)facts.max_sectors_kb, facts.rotational ? ", rotational" : "",
+                         facts.virtio ? ", virtio" : "", (unsigned long long)bytes, depth, adaptive ? " (steered)" : "", stages);
+}
+
 } // namespace
 
 int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
@@ -867,7 +1140,6 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     fstx_config cfg = *cfg_in;
     int rc = normalize(cfg);
     if (rc < 0) return rc;
-    const bool adaptive_depth = (cfg.flags & FSTX_ADAPTIVE_DEPTH) != 0;
 
     int n_dev = fstx_dev::device_count();
     if (n_dev < 0) return n_dev;
@@ -877,14 +1149,11 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 
     std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
     ctx->cfg = cfg;
-    ctx->adaptive_depth = adaptive_depth;
     ctx->no_copy = (cfg.flags & FSTX_PROBE_NO_COPY) != 0;
     ctx->no_read = (cfg.flags & FSTX_PROBE_NO_READ) != 0;
-    ctx->direct_bytes = cfg.direct_read_bytes;
-    ctx->ramp_bytes = std::max(cfg.block_bytes, align_down((uint64_t)cfg.direct_ramp_kb * 1024, cfg.block_bytes));
-    // one staging buffer per read in flight plus one that is being emptied into the ring meanwhile
-    ctx->stage_max = (adaptive_depth ? std::min(cfg.n_threads, 8u) : std::min(cfg.max_direct_reads, cfg.n_threads)) + 1;
-    ctx->direct_gate.reset(new Gate(cfg.max_direct_reads, std::min(cfg.n_threads, 32u), adaptive_depth));
+    ctx->direct_gate.reset(new Gate(1, 1, false));
+    // a configuration that names both depth and size needs no device to settle on
+    if (cfg.max_direct_reads && cfg.direct_read_bytes) settle_direct_shape(ctx.get(), StorageFacts{});
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
 
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
@@ -896,13 +1165,23 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
         // own that binds itself to the node first: the ring is placed there and the caller's
         // affinity and memory policy stay as they are.
         void *p = nullptr;
+        int bound = 0, ring_node = -1;
         std::thread placer([&] {
-            bind_thread_to_node(cfg.numa_node);
+            bound = bind_thread_to_node(cfg.numa_node);
             rc = fstx_dev::set_device(cfg.device_id);
             if (rc == 0) rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
+            if (rc == 0 && p && cfg.numa_node >= 0) {
+                *static_cast<volatile char *>(p) = 0; // the page exists from here on, on the node the policy names
+                ring_node = node_of_address(p);
+            }
         });
         placer.join();
         if (rc < 0) return rc;
+        if (bound < 0) {
+            ctx->ctr.bind_errors.fetch_add(1);
+            ctx->ctr.first_bind_error.store(bound);
+        }
+        ctx->ring_node = ring_node;
         ctx->ring = static_cast<char *>(p);
         fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
     }
@@ -935,9 +1214,12 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
         return rc;
     }
     raw->create_ns = now_ns() - t_start;
-    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu in %.2f ms", cfg.device_id,
+    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu in %.2f ms; node %d: %llu of %u workers on it, "
+                         "ring on node %d, %llu failed bindings (first: %lld)", cfg.device_id,
                          cfg.n_threads, cfg.n_streams, (unsigned long long)cfg.block_bytes,
-                         (unsigned long long)raw->ring_bytes, raw->create_ns / 1e6);
+                         (unsigned long long)raw->ring_bytes, raw->create_ns / 1e6, cfg.numa_node,
+                         (unsigned long long)raw->ctr.workers_on_node.load(), cfg.n_threads, raw->ring_node,
+                         (unsigned long long)raw->ctr.bind_errors.load(), (long long)raw->ctr.first_bind_error.load());
     *out = raw;
     return 0;
 }
@@ -947,7 +1229,7 @@ int fstx_ctx_destroy(fstx_ctx *ctx) {
     const uint64_t t0 = now_ns();
     stop_workers(ctx);
     const uint64_t t1 = now_ns();
-    if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->limit());
+    if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->settled());
     fstx_dev::set_device(ctx->cfg.device_id);
     for (auto s : ctx->streams) fstx_dev::stream_sync(s);
     for (auto &kv : ctx->files) release_file(*kv.second);
@@ -1030,6 +1312,19 @@ int64_t fstx_file_open(fstx_ctx *ctx, const char *path, int mode) {
     if (mode == FSTX_READ_AUTO && f->fd_direct >= 0 && f->size > 0) {
         void *m = mmap(nullptr, f->size, PROT_READ, MAP_SHARED, f->fd_buffered, 0);
         if (m != MAP_FAILED) f->map = m;
+    }
+    if (f->fd_direct >= 0) {
+        // the first file that can be read with O_DIRECT names the device the reads are shaped for
+        bool open_shape;
+        {
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+            open_shape = !ctx->shape_settled;
+        }
+        if (open_shape) {
+            const StorageFacts facts = storage_facts(st.st_dev); // sysfs reads: outside the lock
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+            if (!ctx->shape_settled) settle_direct_shape(ctx, facts);
+        }
     }
     std::lock_guard<std::mutex> lk(ctx->table_mutex);
     int64_t id = ctx->next_file++;
@@ -1115,6 +1410,7 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
                 ctx->queue_bytes += b.len;
                 ctx->queue.push_back(std::move(b));
             }
+            ctx->work_seen.store(true, std::memory_order_release);
         }
         ctx->q_cv.notify_all();
     }
@@ -1197,20 +1493,41 @@ int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request) {
 }
 
 int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
-    if (!ctx || !out) return -FSTX_E_INVAL;
+    // the caller says how large its struct is; a caller built against an older header gets the
+    // fields it knows and nothing is written behind them
+    if (!ctx || !out || out->struct_size < 2 * sizeof(uint64_t)) return -FSTX_E_INVAL;
     const Counters &c = ctx->ctr;
-    out->bounce_buffer_bytes = ctx->ring_bytes;
-    out->bytes_read = c.bytes_read.load();
-    out->bytes_copied = c.bytes_copied.load();
-    out->blocks_buffered = c.blocks_buffered.load();
-    out->blocks_direct = c.blocks_direct.load();
-    out->read_ns = c.read_ns.load();
-    out->stage_ns = c.stage_ns.load();
-    out->slot_wait_ns = c.slot_wait_ns.load();
-    out->direct_fallbacks = c.direct_fallbacks.load();
-    out->direct_depth = ctx->direct_gate->limit();
-    out->direct_reads = c.direct_reads.load();
-    out->create_ns = ctx->create_ns;
+    fstx_metrics m{};
+    m.struct_size = std::min<uint64_t>(out->struct_size, sizeof(fstx_metrics));
+    m.bounce_buffer_bytes = ctx->ring_bytes;
+    m.bytes_read = c.bytes_read.load();
+    m.bytes_copied = c.bytes_copied.load();
+    m.blocks_buffered = c.blocks_buffered.load();
+    m.blocks_direct = c.blocks_direct.load();
+    m.read_ns = c.read_ns.load();
+    m.stage_ns = c.stage_ns.load();
+    m.slot_wait_ns = c.slot_wait_ns.load();
+    m.direct_fallbacks = c.direct_fallbacks.load();
+    m.direct_depth = ctx->direct_gate->settled();
+    m.direct_reads = c.direct_reads.load();
+    m.create_ns = ctx->create_ns;
+    m.numa_node = ctx->cfg.numa_node;
+    m.workers_on_node = c.workers_on_node.load();
+    m.ring_node = ctx->ring_node;
+    m.bind_errors = c.bind_errors.load();
+    m.first_bind_error = c.first_bind_error.load();
+    m.pretouched_bytes = c.pretouched_bytes.load();
+    {
+        std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        m.direct_read_bytes = ctx->shape_settled ? ctx->direct_bytes : 0;
+        m.direct_steered = ctx->shape_settled && ctx->adaptive_depth;
+        m.staging_buffers_max = ctx->shape_settled ? ctx->stage_max : 0;
+        m.storage_nr_requests = ctx->storage.nr_requests;
+        m.storage_max_sectors_kb = ctx->storage.max_sectors_kb;
+        m.storage_flags = (ctx->storage.known ? FSTX_STORAGE_KNOWN : 0) | (ctx->storage.rotational ? FSTX_STORAGE_ROTATIONAL : 0) |
+                          (ctx->storage.virtio ? FSTX_STORAGE_VIRTIO : 0);
+    }
+    std::memcpy(out, &m, (size_t)m.struct_size);
     return 0;
 }
 

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FSTX_ABI_VERSION 2
+#define FSTX_ABI_VERSION 3
 
 /* status codes beyond errno */
 #define FSTX_E_BASE 10000
@@ -68,9 +68,15 @@ typedef struct fstx_config {
     uint32_t n_streams;      /* HIP copy streams shared by the workers (0 = default 4)           */
     uint64_t block_bytes;    /* bytes per read block = per ring slot, multiple of 4096 (0 = 4 MiB)*/
     uint32_t slots_per_thread; /* ring slots each worker cycles through (0 = default 2)          */
-    uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once (0 = default 1)      */
+    uint32_t max_direct_reads; /* O_DIRECT preads allowed in flight at once; 0 = from the block
+                                  device under the first file opened for O_DIRECT: 1 for a
+                                  paravirtual, rotating or unknown disk, else 2 and steered while
+                                  reading (as with FSTX_ADAPTIVE_DEPTH)                          */
     uint64_t direct_read_bytes; /* bytes one O_DIRECT pread covers: a run of consecutive blocks,
-                                   multiple of block_bytes (0 = 1 GiB)                           */
+                                   multiple of block_bytes; 0 = from that device: one request
+                                   queue's worth (nr_requests x max_sectors_kb, 64 MiB .. 1 GiB)
+                                   with one read in flight, a quarter of it with several, and
+                                   never more staging memory than 1/16 of MemAvailable           */
     uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_*                               */
     uint32_t direct_ramp_kb; /* KiB of the first O_DIRECT pread after the queue was empty; the next
                                 ones are 4x, 16x .. as large up to direct_read_bytes, and towards the
@@ -92,8 +98,18 @@ typedef struct fstx_config {
  *            ring -> HBM copies deliver with this engine's slots, streams and threads. */
 #define FSTX_PROBE_NO_COPY 2u
 #define FSTX_PROBE_NO_READ 4u
+/* The workers do not map the pages of their ring slots ahead of the first request (they do by
+ * default: pinned memory is mapped at its first touch, which is slow); for measurements. */
+#define FSTX_NO_PRETOUCH 8u
+
+/* fstx_metrics.storage_flags */
+#define FSTX_STORAGE_KNOWN 1u      /* the block layer named queue depth and request size          */
+#define FSTX_STORAGE_ROTATIONAL 2u
+#define FSTX_STORAGE_VIRTIO 4u
 
 typedef struct fstx_metrics {
+    uint64_t struct_size;         /* in: sizeof(fstx_metrics) of the caller; out: bytes filled in.
+                                     The struct only ever grows at its end.                       */
     uint64_t bounce_buffer_bytes; /* pinned ring bytes currently allocated by this context       */
     uint64_t bytes_read;          /* file bytes delivered into the ring                          */
     uint64_t bytes_copied;        /* bytes enqueued host -> device                               */
@@ -103,14 +119,34 @@ typedef struct fstx_metrics {
     uint64_t stage_ns;            /* summed over workers: staging memcpy after O_DIRECT          */
     uint64_t slot_wait_ns;        /* summed over workers: waiting for a ring slot's last copy    */
     uint64_t direct_fallbacks;    /* blocks that asked for O_DIRECT but were read buffered       */
-    uint64_t direct_depth;        /* O_DIRECT preads currently allowed in flight                 */
+    uint64_t direct_depth;        /* O_DIRECT preads allowed in flight (steered: the depth last
+                                     found good, not a step that is still being tried)           */
     uint64_t direct_reads;        /* O_DIRECT preads issued (each covers a run of blocks)        */
     uint64_t create_ns;           /* what fstx_ctx_create took: threads, ring, streams, events   */
+    /* where the I/O side runs (fstx_config.numa_node >= 0) */
+    int64_t numa_node;            /* the node asked for, -1 = none                               */
+    uint64_t workers_on_node;     /* workers whose CPU affinity, read back with sched_getaffinity
+                                     after binding, lies inside the node's cpulist               */
+    int64_t ring_node;            /* node that holds the ring's first page, -1 where the kernel
+                                     does not say (it does not for device-mapped pinned memory)  */
+    uint64_t bind_errors;         /* threads (workers + the one that allocates the ring) whose
+                                     affinity or memory policy could not be set                  */
+    int64_t first_bind_error;     /* the first such failure as -errno, 0 = none                  */
+    uint64_t pretouched_bytes;    /* ring bytes the workers mapped before the first request      */
+    /* the O_DIRECT reads as settled (0 until a file has been opened for O_DIRECT) */
+    uint64_t direct_read_bytes;   /* bytes one read covers                                       */
+    uint64_t direct_steered;      /* 1 = direct_depth is steered while reading                   */
+    uint64_t staging_buffers_max; /* staging buffers of direct_read_bytes the context may hold   */
+    uint64_t storage_nr_requests; /* /sys/dev/block/<dev>/queue/nr_requests of that file's device */
+    uint64_t storage_max_sectors_kb;
+    uint64_t storage_flags;       /* FSTX_STORAGE_*                                              */
 } fstx_metrics;
 
 /* ---- library-wide helpers ------------------------------------------------ */
 
-/* ABI version of the loaded library (FSTX_ABI_VERSION). */
+/* ABI version of the loaded library (FSTX_ABI_VERSION).  Call it first and compare it with the
+ * FSTX_ABI_VERSION the caller was built against: structs passed by pointer carry their size
+ * (fstx_config, fstx_metrics), everything else is only guaranteed within one version. */
 int fstx_abi_version(void);
 
 /* Number of visible HIP devices, or -FSTX_E_NO_DEVICE.
@@ -124,8 +160,16 @@ int fstx_get_alignment_size(void);
 int fstx_get_device_pci_bus(int device_id, char *out, int len);
 
 /* Restrict the calling thread (and threads it creates later) to the CPUs of a
- * NUMA node and prefer its memory.  set_numa_node (cpp/ext.cpp:525-533). */
+ * NUMA node and prefer its memory.  0, or what failed as -errno (-ENODEV: the node has no
+ * CPUs or does not exist).  set_numa_node (cpp/ext.cpp:525-533). */
 int fstx_set_numa_node(int numa_node);
+
+/* The CPUs of a NUMA node as the library reads them from sysfs
+ * (<root>/devices/system/node/node<N>/cpulist, root = /sys or $FSTX_SYSFS_ROOT): up to
+ * `capacity` of them into cpus[], ascending; returns how many the node has, or -ENODEV.
+ * The I/O workers of a context with numa_node = N are bound to exactly these.  Stands in
+ * for libnuma's node-to-CPU lookup behind numa_run_on_node (cpp/ext.cpp:525-533). */
+int fstx_node_cpus(int numa_node, int *cpus, int capacity);
 
 /* Toggle debug lines on stderr.  set_debug_log (cpp/ext.cpp:417-420). */
 void fstx_set_debug_log(int enabled);
@@ -196,7 +240,8 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
  * nogds_file_reader::wait_read (cpp/ext.cpp:765-776). */
 int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request);
 
-/* Snapshot of the context's counters. */
+/* Snapshot of the context's counters.  Set out->struct_size = sizeof(fstx_metrics) before the
+ * call: the library fills in at most that many bytes and stores the count it filled. */
 int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out);
 
 /* ---- HBM kernels ----------------------------------------------------------- */

@@ -94,7 +94,19 @@ int main(int argc, char **argv) {
         CHECK(fstx_file_close(ctx, file) == 0);
     }
     fstx_metrics met;
-    CHECK(fstx_get_metrics(ctx, &met) == 0 && met.bytes_copied >= 3 * (size - 10));
+    memset(&met, 0, sizeof met);
+    met.struct_size = sizeof met;
+    CHECK(fstx_get_metrics(ctx, &met) == 0 && met.bytes_copied >= 3 * (size - 10) && met.struct_size == sizeof met);
+    {
+        /* a caller built against a shorter struct: the library fills what fits and not a byte more */
+        uint64_t old_caller[8];
+        memset(old_caller, 0xEE, sizeof old_caller);
+        old_caller[0] = 4 * sizeof(uint64_t);
+        CHECK(fstx_get_metrics(ctx, (fstx_metrics *)old_caller) == 0);
+        CHECK(old_caller[0] == 4 * sizeof(uint64_t) && old_caller[2] == met.bytes_read && old_caller[4] == 0xEEEEEEEEEEEEEEEEull);
+        int cpus[4];
+        CHECK(fstx_node_cpus(-1, cpus, 4) < 0);
+    }
     CHECK(fstx_ctx_destroy(ctx) == 0);
     CHECK(fstx_bounce_buffer_bytes() == 0);
 

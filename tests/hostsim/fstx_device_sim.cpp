@@ -79,6 +79,16 @@ struct SimStream {
     }
 };
 
+// Storage model behind the O_DIRECT reads of the pipeline (fstx_test_after_direct_read): up to
+// `parallel` requests are served at once, each at bandwidth / parallel, after a fixed latency.
+struct StorageModel {
+    std::mutex m;
+    std::condition_variable cv;
+    int lat_us = 0, parallel = 0, busy = 0;
+    double bytes_per_us = 0; // of one channel
+};
+StorageModel g_storage;
+
 std::atomic<int> g_copy_delay_us{50};
 std::atomic<int64_t> g_fail_copy_after{-1};
 std::atomic<int64_t> g_pinned_live{0};
@@ -88,6 +98,27 @@ std::atomic<int64_t> g_pinned_live{0};
 extern "C" {
 // knobs for the tests
 void fstx_sim_set_copy_delay_us(int us) { g_copy_delay_us.store(us); }
+// parallel = 0 switches the model off
+void fstx_sim_set_storage(int lat_us, double bandwidth_MBps, int parallel) {
+    std::lock_guard<std::mutex> lk(g_storage.m);
+    g_storage.lat_us = lat_us;
+    g_storage.parallel = parallel;
+    g_storage.bytes_per_us = parallel > 0 ? bandwidth_MBps / parallel : 0; // MB/s = bytes/us
+}
+// the pipeline calls this after every O_DIRECT pread (a weak symbol there, defined only here)
+void fstx_test_after_direct_read(uint64_t bytes) {
+    std::unique_lock<std::mutex> lk(g_storage.m);
+    if (g_storage.parallel <= 0) return;
+    g_storage.cv.wait(lk, [] { return g_storage.busy < g_storage.parallel; });
+    ++g_storage.busy;
+    const double us = g_storage.lat_us + (g_storage.bytes_per_us > 0 ? bytes / g_storage.bytes_per_us : 0);
+    lk.unlock();
+    std::this_thread::sleep_for(std::chrono::microseconds((long long)us));
+    lk.lock();
+    --g_storage.busy;
+    lk.unlock();
+    g_storage.cv.notify_one();
+}
 void fstx_sim_fail_copy_after(int64_t n) { g_fail_copy_after.store(n); }
 int64_t fstx_sim_pinned_live(void) { return g_pinned_live.load(); }
 // a caller-side stream: created here, handed to fstx_ctx_order_after as its `stream`

@@ -49,7 +49,7 @@ int main(int argc, char **argv) {
         fstx_config cfg{};
         cfg.struct_size = sizeof cfg;
         cfg.device_id = 0;
-        cfg.numa_node = -1;
+        cfg.numa_node = round == 1 ? 0 : -1; // one round with the workers bound to a node and the ring placed on it
         cfg.n_threads = 2 + round * 3;
         cfg.n_streams = 1 + round;
         cfg.block_bytes = 4096u << (round * 2);
@@ -96,7 +96,8 @@ int main(int argc, char **argv) {
             });
         }
         for (auto &t : callers) t.join();
-        fstx_metrics m;
+        fstx_metrics m{};
+        m.struct_size = sizeof m;
         fstx_get_metrics(ctx, &m);
         if (m.bytes_copied != 3 * size) bad++;
         fstx_sim_stream_destroy(foreign); // drains it: the stand-in's events must outlive their records
