@@ -337,12 +337,12 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int) -> dict:
         drop_cache(files)
         return run_load(files, "auto", threads, 4096, None, **kw)
 
-    def leg(probe, cold):
+    def leg(probe, cold, reps=3, **kw):
         rates = []
-        for _ in range(3):
+        for _ in range(reps):
             if cold:
                 drop_cache(files)
-            rates.append(engine_leg(files, probe, threads, 4096))
+            rates.append(engine_leg(files, probe, threads, 4096, **kw))
         return max(rates, key=lambda r: r["GBps"])
 
     ro = leg("read_only", True)
@@ -353,17 +353,30 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int) -> dict:
     out["cold"]["read_only_leg_GBps"] = ro["GBps"]
     out["cold"]["io_over_read_only_leg"] = out["cold"]["io_s"] / ro["seconds"]
     warm_cache(files)
-    co = leg("copy_only", False)
-    co_held = max((engine_leg(files, "copy_only", threads, 4096, held=True) for _ in range(3)), key=lambda r: r["GBps"])
-    out["warm"] = best(lambda: run_load(files, "auto", threads, 4096, None), reps=5)
+    # warm: loads and legs take turns (the box's link rate drifts by 10-20 % within seconds), best of each
+    variants = {"warm": {}}
+    if key == "C2":
+        variants["warm_window_layout_realign"] = {"layout": "window"}
+    loads = {k: [] for k in variants}
+    legs = []
+    for _ in range(4):
+        legs.append(leg("copy_only", False, reps=2))
+        for k, kw in variants.items():
+            loads[k] += [run_load(files, "auto", threads, 4096, None, **kw) for _ in range(2)]
+    co = max(legs, key=lambda r: r["GBps"])
+    for k in variants:
+        out[k] = best(lambda it=iter(loads[k]): next(it), reps=len(loads[k]))
     hold = hold_reader("cuda:0", max_threads=threads, block_size_kb=4096)
     try:
         run_load(files, "auto", threads, 4096, None)  # maps the ring's pages
-        out["warm_held_reader"] = best(lambda: run_load(files, "auto", threads, 4096, None), reps=5)
+        held_loads, held_legs = [], []
+        for _ in range(3):
+            held_legs.append(leg("copy_only", False, reps=2, held=True))
+            held_loads += [run_load(files, "auto", threads, 4096, None) for _ in range(2)]
+        co_held = max(held_legs, key=lambda r: r["GBps"])
+        out["warm_held_reader"] = best(lambda it=iter(held_loads): next(it), reps=len(held_loads))
     finally:
         hold.close()
-    if key == "C2":
-        out["warm_window_layout_realign"] = best(lambda: run_load(files, "auto", threads, 4096, None, layout="window"), reps=5)
     for k in ("warm", "warm_held_reader", "warm_window_layout_realign"):
         if k in out:
             # a load under a held reader is compared with the leg of an engine that existed before, too

@@ -445,7 +445,8 @@ class Reader:
     ``shared=True`` asks the library for the process-wide context of this configuration
     (``fstx_ctx_acquire``): readers that are alive at the same time then use one set of
     threads, one ring and one set of streams, and the last ``close`` frees them.
-    ``probe`` is ``PROBE_NO_COPY`` or ``PROBE_NO_READ`` for a measurement context.
+    ``probe`` is ``PROBE_NO_COPY`` or ``PROBE_NO_READ`` for a measurement context;
+    ``pretouch=False`` keeps the workers from mapping their ring slots ahead of the first request.
     """
 
     def __init__(
@@ -462,11 +463,12 @@ class Reader:
         direct_ramp_kb: int = 0,
         probe: int = 0,
         shared: bool = False,
+        pretouch: bool = True,
     ):
         cfg = FstxConfig(
             ctypes.sizeof(FstxConfig), device_id, numa_node, n_threads, n_streams, block_bytes,
             slots_per_thread, max_direct_reads, direct_read_bytes,
-            (ADAPTIVE_DEPTH if adaptive_depth else 0) | probe, direct_ramp_kb,
+            (ADAPTIVE_DEPTH if adaptive_depth else 0) | probe | (0 if pretouch else NO_PRETOUCH), direct_ramp_kb,
         )
         handle = ctypes.c_void_p()
         self._shared = shared

@@ -86,6 +86,7 @@ def _check_header_size(n: int, buffer_len: int, where: str) -> None:
 
 
 Index = Union[int, slice]
+_DTYPE_OF_TAG = {d.value: d for d in DType}
 
 
 @dataclass
@@ -106,17 +107,18 @@ class TensorFrame:
     @classmethod
     def from_buffer(cls, entry: Dict[str, Any]) -> "TensorFrame":
         shape = entry["shape"]
-        strides = [1] * len(shape)
-        for d in range(len(shape) - 2, -1, -1):
-            strides[d] = strides[d + 1] * shape[d + 1]
-        return cls(
-            DType(entry["dtype"]),
-            shape,
-            list(entry["data_offsets"]),
-            strides,
-            [0] * len(shape),
-            False,
-        )
+        rank = len(shape)
+        if rank == 2:  # most tensors of a checkpoint
+            strides = [shape[1], 1]
+        else:
+            strides = [1] * rank
+            for d in range(rank - 2, -1, -1):
+                strides[d] = strides[d + 1] * shape[d + 1]
+        tag = entry["dtype"]
+        dtype = _DTYPE_OF_TAG.get(tag)
+        if dtype is None:
+            dtype = DType(tag)  # raises for an unknown tag, as the enum does
+        return cls(dtype, shape, list(entry["data_offsets"]), strides, [0] * rank, False)
 
     def __repr__(self) -> str:
         return str({"dtype": self.dtype, "shape": self.shape, "data_offsets": self.data_offsets})
@@ -181,7 +183,7 @@ class SafeTensorsMetadata:
         self.framework = framework
         self.header_length = header_length
         self.size_bytes = size_bytes
-        table = json.loads(string, object_pairs_hook=OrderedDict)
+        table = json.loads(string)  # a plain dict keeps the file's key order (and parses in C throughout)
         self.metadata = table.pop("__metadata__", "") or ""
         if keep_orig_dict:
             self.ser = table
@@ -190,7 +192,11 @@ class SafeTensorsMetadata:
 
         self.tensors: Dict[str, TensorFrame] = {}
         cursor = 0
-        for name, entry in sorted(table.items(), key=lambda kv: kv[1]["data_offsets"][0]):
+        items = list(table.items())
+        starts = [entry["data_offsets"][0] for _, entry in items]
+        if any(a > b for a, b in zip(starts, starts[1:])):  # writers emit them in offset order; sort only when not
+            items.sort(key=lambda kv: kv[1]["data_offsets"][0])
+        for name, entry in items:
             frame = TensorFrame.from_buffer(entry)
             begin, end = frame.data_offsets
             if begin != cursor or end < begin:

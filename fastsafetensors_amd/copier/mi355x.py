@@ -31,7 +31,8 @@ Arena layouts
 """
 
 import os
-from typing import Dict, List, Optional, Tuple
+import threading
+from typing import Callable, Dict, List, Optional, Tuple
 
 from .. import _native
 from ..common import SafeTensorsMetadata, TensorFrame
@@ -136,29 +137,21 @@ class MI355XFileCopier(CopierInterface):
     def wait_io(
         self, gbuf: _native.DeviceBuffer, dtype: DType = DType.AUTO, noalign: bool = False
     ) -> Dict[str, TensorBase]:
-        failed = self._drain()
-        if failed:
-            raise Exception(
-                f"wait_io: read failed, file={self.metadata.src}, "
-                + ", ".join(f"req {r}: {e}" for r, e in failed)
-            )
         meta, fw = self.metadata, self.framework
-        arena, data_at = gbuf, self.data_at
         if dtype != DType.AUTO and any(f.dtype != dtype for f in meta.tensors.values()):
+            self._drain_or_raise()
             return self._converted(gbuf, dtype)
+
+        # Everything that does not need the bytes happens while they are still on their way: where
+        # each tensor will live, the side allocations, and the views (hundreds per file -- as long
+        # as the transfer of a small file's last tenth).  The kernels follow the wait.
+        arena, data_at = gbuf, self.data_at
+        shift_from = None
         if self.layout == "window" and not noalign and data_at % PTR_ALIGN and meta.data_length:
-            # shift the whole data section onto a 16-byte boundary, out of place
+            # the whole data section will be shifted onto a 16-byte boundary, out of place
             lead = pick_lead(list(meta.tensors.values()))
             fresh = fw.alloc_side_memory(gbuf, lead + meta.data_length, self.device)
-            _native.realign_copy(
-                fresh.get_base_address() + lead,
-                gbuf.get_base_address() + data_at,
-                meta.data_length,
-                self._stream(),
-            )
-            # the window goes back to the allocator right away: its reuse is ordered after this
-            # kernel on the same stream, and by order_after() for the copy streams
-            fw.shrink_tensor_memory(gbuf)
+            shift_from = (gbuf.get_base_address() + data_at, fresh.get_base_address() + lead)
             arena, data_at = fresh, lead
 
         # tensors that still start off-boundary move to an aligned side buffer
@@ -176,6 +169,19 @@ class MI355XFileCopier(CopierInterface):
                 placed[name] = cursor
                 cursor += _align_up(frame.nbytes, LINE_ALIGN)
             side = fw.alloc_side_memory(gbuf, cursor, self.device)
+        in_arena = [(n, data_at + f.data_offsets[0], f) for n, f in meta.tensors.items() if n not in placed]
+        views = fw.view_tensors(arena, in_arena, self.device)
+        if placed:
+            views.update(fw.view_tensors(side, [(n, placed[n], meta.tensors[n]) for n in placed], self.device))
+        tensors = {name: views[name] for name in meta.tensors}  # in the file's order
+
+        self._drain_or_raise()
+        if shift_from is not None:
+            _native.realign_copy(shift_from[1], shift_from[0], meta.data_length, self._stream())
+            # the window goes back to the allocator right away: its reuse is ordered after this
+            # kernel on the same stream, and by order_after() for the copy streams
+            fw.shrink_tensor_memory(gbuf)
+        if need:
             _native.realign_copy_batch(
                 [
                     (side.get_base_address() + placed[n], base + data_at + f.data_offsets[0], f.nbytes)
@@ -183,12 +189,15 @@ class MI355XFileCopier(CopierInterface):
                 ],
                 self._stream(),
             )
+        return tensors
 
-        in_arena = [(n, data_at + f.data_offsets[0], f) for n, f in meta.tensors.items() if n not in placed]
-        views = fw.view_tensors(arena, in_arena, self.device)
-        if placed:
-            views.update(fw.view_tensors(side, [(n, placed[n], meta.tensors[n]) for n in placed], self.device))
-        return {name: views[name] for name in meta.tensors}  # in the file's order
+    def _drain_or_raise(self) -> None:
+        failed = self._drain()
+        if failed:
+            raise Exception(
+                f"wait_io: read failed, file={self.metadata.src}, "
+                + ", ".join(f"req {r}: {e}" for r, e in failed)
+            )
 
     def _converted(self, gbuf: _native.DeviceBuffer, dtype: DType) -> Dict[str, TensorBase]:
         """Tensors down-cast to ``dtype`` on the GPU (``common.py:355-375`` does it with
@@ -295,7 +304,7 @@ def _default_numa_node(device: Device) -> int:
     return -1 if node is None or node < 0 else node
 
 
-def _open_reader(
+def _reader_settings(
     device: Device,
     max_threads: int = 16,
     block_size_kb: Optional[int] = None,
@@ -307,11 +316,13 @@ def _open_reader(
     adaptive_depth: bool = False,
     numa_node: Optional[int] = None,
     shared_reader: bool = True,
-) -> _native.Reader:
+    pretouch: bool = True,
+) -> Dict[str, int]:
+    """Arguments of ``_native.Reader`` from the copier's own, defaults and environment resolved."""
     block_kb = block_size_kb or int(os.environ.get("FSTX_BLOCK_KB", "4096"))
-    return _native.Reader(
-        device.index if device.index is not None else 0,
-        numa_node=_default_numa_node(device) if numa_node is None else numa_node,
+    return dict(
+        device_id=device.index if device.index is not None else 0,
+        numa_node=numa_node,  # None: looked up from the device (a sysfs read) by whoever builds the reader
         n_threads=max_threads,
         n_streams=n_streams,
         block_bytes=block_kb * 1024,
@@ -321,7 +332,60 @@ def _open_reader(
         adaptive_depth=adaptive_depth,
         direct_ramp_kb=direct_ramp_kb if direct_ramp_kb is not None else int(os.environ.get("FSTX_DIRECT_RAMP_KB", "0")),
         shared=shared_reader,
+        pretouch=pretouch,
     )
+
+
+def _build_reader(device: Device, settings: Dict[str, int]) -> _native.Reader:
+    if settings["numa_node"] is None:
+        settings = dict(settings, numa_node=_default_numa_node(device))
+    return _native.Reader(**settings)
+
+
+def _open_reader(device: Device, **kwargs) -> _native.Reader:
+    return _build_reader(device, _reader_settings(device, **kwargs))
+
+
+class DeferredReader:
+    """A ``_native.Reader`` that is being built on a helper thread.
+
+    Building one takes a millisecond or two (threads, streams, events, the pinned ring) and needs
+    nothing from the caller, who has file headers to parse meanwhile; the first use of the reader
+    joins the helper.  Every attribute is the real reader's; an error of the build is raised at
+    that first use (``wait()`` raises it on demand)."""
+
+    def __init__(self, build: Callable[[], _native.Reader]):
+        self._reader: Optional[_native.Reader] = None
+        self._error: Optional[BaseException] = None
+        self._thread: Optional[threading.Thread] = threading.Thread(
+            target=self._run, args=(build,), name="fstx-reader-create", daemon=True
+        )
+        self._thread.start()
+
+    def _run(self, build: Callable[[], _native.Reader]) -> None:
+        try:
+            self._reader = build()
+        except BaseException as e:  # handed to the thread that uses the reader
+            self._error = e
+
+    def wait(self) -> _native.Reader:
+        t = self._thread
+        if t is not None:
+            t.join()
+            self._thread = None
+        if self._error is not None:
+            raise self._error
+        return self._reader
+
+    def __getattr__(self, name):
+        return getattr(self.wait(), name)
+
+    def close(self) -> None:
+        t, self._thread = self._thread, None
+        if t is not None:
+            t.join()
+        if self._reader is not None:
+            self._reader.close()
 
 
 def hold_reader(device: str = "cuda:0", max_threads: int = 16, **kwargs) -> _native.Reader:
@@ -358,6 +422,7 @@ def new_mi355x_file_copier(
     adaptive_depth: bool = False,
     numa_node: Optional[int] = None,
     shared_reader: bool = True,
+    pretouch: bool = True,
     **kwargs,
 ) -> CopierConstructFunc:
     """One read pipeline (threads, pinned ring, streams) shared by every file of a
@@ -376,11 +441,13 @@ def new_mi355x_file_copier(
         raise Exception("[FAIL] no HIP device is visible to libfstx")
     read_mode = read_mode or os.environ.get("FSTX_READ_MODE", "auto")
     layout = layout or os.environ.get("FSTX_LAYOUT", "direct")
-    reader = _open_reader(
+    settings = _reader_settings(
         device, max_threads=max_threads, block_size_kb=block_size_kb, n_streams=n_streams,
         slots_per_thread=slots_per_thread, max_direct_reads=max_direct_reads, direct_read_kb=direct_read_kb,
-        direct_ramp_kb=direct_ramp_kb, adaptive_depth=adaptive_depth, numa_node=numa_node, shared_reader=shared_reader,
+        direct_ramp_kb=direct_ramp_kb, adaptive_depth=adaptive_depth, numa_node=numa_node, shared_reader=shared_reader, pretouch=pretouch,
     )
+    # built on a helper thread: the caller goes on to parse headers and joins it at the first file
+    reader = DeferredReader(lambda: _build_reader(device, settings))
 
     def construct(metadata: SafeTensorsMetadata, device: Device, framework: FrameworkOpBase) -> CopierInterface:
         return MI355XFileCopier(metadata, device, reader, framework, read_mode=read_mode, layout=layout)

@@ -61,6 +61,8 @@ namespace {
 
 constexpr uint64_t kPage = 4096;
 constexpr uint64_t kDefaultBlock = 4ull << 20;
+constexpr uint64_t kSmallRequestBlock = 1ull << 20;  // block size for requests under kSmallRequest
+constexpr uint64_t kSmallRequest = 2ull << 30;
 constexpr double kResidentEnough = 0.95;
 
 inline uint64_t align_down(uint64_t v, uint64_t a) { return v - v % a; }
@@ -428,6 +430,10 @@ struct fstx_ctx {
     bool head_wants_direct = false;        // whether the block at the head of `queue` is to be read with O_DIRECT
     bool extending = false;                // a worker asks the page cache how far its run may reach: `queue` is its alone meanwhile
     bool closing = false;
+    // Workers that take work (q_mutex).  A small request on an idle context wakes only half of
+    // them: every slot that is used for the first time costs its first touch, and eight workers
+    // keep the link as busy as sixteen; anything larger, or more work behind it, wakes all.
+    uint32_t active_workers = 0;
     std::atomic<bool> work_seen{false};    // something was queued at least once: the workers stop touching their idle slots
 
     std::mutex done_mutex;
@@ -774,23 +780,35 @@ struct Worker {
         return 0;
     }
 
-    // Map the pages of this worker's idle slots into the process before the first block needs
-    // them: pinned memory is mapped page by page at its first touch, and that costs more per
-    // byte than copying it to the device (measured 0.34 ms per MiB on one thread, 0.06 with
-    // sixteen).  Runs while the creating thread still builds the rest of the context and its
-    // caller parses file headers, and stops for good as soon as anything is queued -- from
-    // then on the reads touch what is left as they go, and a slot may hold data.
-    void pretouch() {
+    // Map the ring's pages into the process before the first block needs them: pinned memory
+    // is mapped page by page at its first touch, and that costs more per byte than copying it
+    // to the device (measured: 0.34 ms per MiB on one thread, 0.06 with eight or more, i.e.
+    // 18 GB/s at best against a 57 GB/s link).  A few of the workers do it -- more gain nothing,
+    // and the creating thread and its caller must still find a free CPU -- by READING one byte
+    // per page, which is harmless to a slot that is already in use.  The part of every slot that
+    // the blocks of small requests use comes first.  Runs while the creating thread builds the
+    // rest of the context and its caller parses file headers, and stops as soon as anything is
+    // queued: from then on the reads touch what is left as they go.
+    void pretouch(uint32_t helpers) {
+        const uint64_t slots = (uint64_t)ctx->cfg.n_threads * ctx->cfg.slots_per_thread;
+        const uint64_t head = std::min(ctx->slot_bytes, kSmallRequestBlock + kPage);
         uint64_t done = 0;
-        for (Slot &slot : *mine)
-            for (uint64_t at = 0; at < ctx->slot_bytes; at += kPage) {
-                if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
-                    ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
-                    return;
+        char sink = 0;
+        for (int pass = 0; pass < 2; ++pass) {
+            const uint64_t from = pass == 0 ? 0 : head, to = pass == 0 ? head : ctx->slot_bytes;
+            for (uint64_t s = index; s < slots; s += helpers) {
+                const char *base = ctx->ring + s * ctx->slot_bytes;
+                for (uint64_t at = from; at < to; at += kPage) {
+                    if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
+                        ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
+                        return;
+                    }
+                    sink ^= *(const volatile char *)(base + at);
+                    done += kPage;
                 }
-                *(volatile char *)(slot.host + at) = 0;
-                done += kPage;
             }
+        }
+        (void)sink;
         ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
     }
 
@@ -816,7 +834,10 @@ struct Worker {
         ctx->ready_cv.notify_all();
         stream_ix = index % (uint32_t)ctx->streams.size();
         stream = ctx->streams[stream_ix];
-        if (dev_rc == 0 && !ctx->no_read && !(ctx->cfg.flags & FSTX_NO_PRETOUCH)) pretouch();
+        if (dev_rc == 0 && !ctx->no_read && !(ctx->cfg.flags & FSTX_NO_PRETOUCH)) {
+            const uint32_t helpers = std::min(std::min(ctx->cfg.n_threads, 8u), std::max(1u, std::thread::hardware_concurrency() / 2));
+            if (index < helpers) pretouch(helpers);
+        }
         std::vector<Block> run;
         std::vector<int64_t> status;
         for (;;) {
@@ -839,6 +860,7 @@ struct Worker {
                 for (;;) {
                     // (while another worker extends its run, the queue is that worker's alone)
                     ctx->q_cv.wait(lk, [&] {
+                        if (index >= ctx->active_workers && !ctx->closing) return false; // not needed for what is queued
                         return !ctx->staged.empty() || (!ctx->extending && (ctx->closing || !ctx->queue.empty()));
                     });
                     if (ctx->extending || ctx->queue.empty()) {
@@ -854,6 +876,12 @@ struct Worker {
                         ctx->head_wants_direct = dev_rc == 0 && head.req->error.load(std::memory_order_relaxed) == 0 &&
                                                  wants_direct(head);
                         ctx->head_verdict_for = ctx->queue_pops;
+                        // O_DIRECT reads want everybody: each one in flight holds a worker, and what
+                        // they stage is copied out by all the others
+                        if (ctx->head_wants_direct && ctx->active_workers < ctx->cfg.n_threads) {
+                            ctx->active_workers = ctx->cfg.n_threads;
+                            woke_others = true;
+                        }
                     }
                     direct = ctx->head_wants_direct;
                     if (!direct) break; // a page-cache block: read it now
@@ -1384,11 +1412,12 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
     // first byte, so that every block's O_DIRECT window fits one slot.
     std::vector<Block> blocks;
     if (length && req->error.load() == 0) {
-        // Small requests are cut into smaller blocks (at least 512 KiB, about 256 per request):
-        // a slot's pages are mapped at their first touch, which is slow for pinned memory, and a
-        // small load would otherwise spend longer touching the whole ring than copying.
+        // Requests under 2 GiB are cut into blocks of 1 MiB: a slot's pages are mapped at their
+        // first touch, at 18 GB/s at best, so a load moves at that rate until the part of the ring
+        // it uses has been touched once -- 2.5 ms for 32 slots of 2 MiB, which is a sixth of a
+        // 0.7 GB load.  1 MiB blocks still run the link at 56 of its 57 GB/s.
         uint64_t bb = ctx->cfg.block_bytes;
-        while (bb > (512u << 10) && bb % (2 * kPage) == 0 && bb * 256 > length) bb /= 2;
+        if (length < kSmallRequest) bb = std::min(bb, kSmallRequestBlock);
         const uint64_t origin = align_down(file_off, kPage);
         const uint64_t end = file_off + length;
         for (uint64_t lo = origin; lo < end; lo += bb) {
@@ -1406,6 +1435,9 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
                 req->file->open_requests.fetch_sub(1);
                 return -FSTX_E_CLOSED;
             }
+            const bool idle = ctx->queue.empty() && ctx->staged.empty();
+            const uint32_t all = ctx->cfg.n_threads;
+            ctx->active_workers = idle && length < kSmallRequest ? std::min(all, std::max(4u, all / 2)) : all;
             for (Block &b : blocks) {
                 ctx->queue_bytes += b.len;
                 ctx->queue.push_back(std::move(b));

@@ -134,9 +134,11 @@ def test_shared_reader_lives_as_long_as_someone_holds_it(golden):
     path = golden("a.safetensors")
     ring = 4 * 2 * (4096 * 1024 + 4096)
     a = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)
+    a.copier_constructor.reader.wait()  # a loader's reader is built on a helper thread; wait() joins it
     assert _native.bounce_buffer_bytes() == ring
     b = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)          # same settings: same reader
     c = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4, shared_reader=False)
+    b.copier_constructor.reader.wait(), c.copier_constructor.reader.wait()
     assert _native.bounce_buffer_bytes() == 2 * ring
     for ld in (a, b, c):
         ld.add_filenames({0: [path]})
