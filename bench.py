@@ -232,7 +232,8 @@ def engine_leg(files: List[str], probe: str, threads: int, block_kb: int, read_m
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         if reader is None:
-            reader = _native.Reader(0, n_threads=threads, block_bytes=block_kb * 1024, probe=flag, shared=False)
+            reader = _native.Reader(0, n_threads=threads, block_bytes=block_kb * 1024, probe=flag, shared=False,
+                                    async_create=True)
         handles, reqs = [], []
         for path, meta, arena, n in zip(files, metas, arenas, sizes):
             h = reader.open(path, mode)

@@ -24,6 +24,7 @@ READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
 ADAPTIVE_DEPTH = 1
 PROBE_NO_COPY, PROBE_NO_READ = 2, 4
 NO_PRETOUCH = 8
+CREATE_ASYNC = 16
 STORAGE_KNOWN, STORAGE_ROTATIONAL, STORAGE_VIRTIO = 1, 2, 4
 READ_MODES = {"auto": READ_AUTO, "buffered": READ_BUFFERED, "direct": READ_DIRECT}
 
@@ -447,6 +448,9 @@ class Reader:
     threads, one ring and one set of streams, and the last ``close`` frees them.
     ``probe`` is ``PROBE_NO_COPY`` or ``PROBE_NO_READ`` for a measurement context;
     ``pretouch=False`` keeps the workers from mapping their ring slots ahead of the first request.
+    ``async_create=True``: the constructor returns once the settings are checked and the library
+    builds threads, streams and ring meanwhile; ``wait_read`` / ``metrics`` wait for that build
+    and report its failure.
     """
 
     def __init__(
@@ -464,11 +468,13 @@ class Reader:
         probe: int = 0,
         shared: bool = False,
         pretouch: bool = True,
+        async_create: bool = False,
     ):
         cfg = FstxConfig(
             ctypes.sizeof(FstxConfig), device_id, numa_node, n_threads, n_streams, block_bytes,
             slots_per_thread, max_direct_reads, direct_read_bytes,
-            (ADAPTIVE_DEPTH if adaptive_depth else 0) | probe | (0 if pretouch else NO_PRETOUCH), direct_ramp_kb,
+            (ADAPTIVE_DEPTH if adaptive_depth else 0) | probe | (0 if pretouch else NO_PRETOUCH)
+            | (CREATE_ASYNC if async_create else 0), direct_ramp_kb,
         )
         handle = ctypes.c_void_p()
         self._shared = shared

@@ -31,8 +31,7 @@ Arena layouts
 """
 
 import os
-import threading
-from typing import Callable, Dict, List, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 from .. import _native
 from ..common import SafeTensorsMetadata, TensorFrame
@@ -346,48 +345,6 @@ def _open_reader(device: Device, **kwargs) -> _native.Reader:
     return _build_reader(device, _reader_settings(device, **kwargs))
 
 
-class DeferredReader:
-    """A ``_native.Reader`` that is being built on a helper thread.
-
-    Building one takes a millisecond or two (threads, streams, events, the pinned ring) and needs
-    nothing from the caller, who has file headers to parse meanwhile; the first use of the reader
-    joins the helper.  Every attribute is the real reader's; an error of the build is raised at
-    that first use (``wait()`` raises it on demand)."""
-
-    def __init__(self, build: Callable[[], _native.Reader]):
-        self._reader: Optional[_native.Reader] = None
-        self._error: Optional[BaseException] = None
-        self._thread: Optional[threading.Thread] = threading.Thread(
-            target=self._run, args=(build,), name="fstx-reader-create", daemon=True
-        )
-        self._thread.start()
-
-    def _run(self, build: Callable[[], _native.Reader]) -> None:
-        try:
-            self._reader = build()
-        except BaseException as e:  # handed to the thread that uses the reader
-            self._error = e
-
-    def wait(self) -> _native.Reader:
-        t = self._thread
-        if t is not None:
-            t.join()
-            self._thread = None
-        if self._error is not None:
-            raise self._error
-        return self._reader
-
-    def __getattr__(self, name):
-        return getattr(self.wait(), name)
-
-    def close(self) -> None:
-        t, self._thread = self._thread, None
-        if t is not None:
-            t.join()
-        if self._reader is not None:
-            self._reader.close()
-
-
 def hold_reader(device: str = "cuda:0", max_threads: int = 16, **kwargs) -> _native.Reader:
     """Keep the process-wide read pipeline of this configuration alive until the returned
     handle is closed.
@@ -446,8 +403,9 @@ def new_mi355x_file_copier(
         slots_per_thread=slots_per_thread, max_direct_reads=max_direct_reads, direct_read_kb=direct_read_kb,
         direct_ramp_kb=direct_ramp_kb, adaptive_depth=adaptive_depth, numa_node=numa_node, shared_reader=shared_reader, pretouch=pretouch,
     )
-    # built on a helper thread: the caller goes on to parse headers and joins it at the first file
-    reader = DeferredReader(lambda: _build_reader(device, settings))
+    # the library builds threads, streams and the ring behind this call's back (a millisecond,
+    # during which the caller parses headers, opens files and queues reads)
+    reader = _build_reader(device, dict(settings, async_create=True))
 
     def construct(metadata: SafeTensorsMetadata, device: Device, framework: FrameworkOpBase) -> CopierInterface:
         return MI355XFileCopier(metadata, device, reader, framework, read_mode=read_mode, layout=layout)

@@ -439,11 +439,26 @@ struct fstx_ctx {
     std::mutex done_mutex;
     std::condition_variable done_cv;
 
-    // start-up handshake: every worker reports once its slots and events exist
+    // start-up handshake (ready_mutex): the workers are started first and make their events while
+    // the ring is allocated and the streams are created; `parts_ready` releases them, and every
+    // worker reports once its slots exist.  `built` closes the build; a failed one leaves its
+    // status in `build_status` and in `failed` (q_mutex), the workers count off whatever is queued.
     std::mutex ready_mutex;
     std::condition_variable ready_cv;
     uint32_t ready = 0;
     int ready_status = 0;
+    bool ring_ready = false;      // the ring's fate is known (it exists, or parts_status says why not)
+    bool parts_ready = false;
+    std::unique_ptr<std::atomic<uint8_t>[]> head_mapped; // per ring slot: its owner has mapped the head already
+    std::atomic<bool> parts_seen{false}; // parts_ready, for the workers that map their slots meanwhile
+    int parts_status = 0;
+    bool built = false;
+    int build_status = 0;
+    std::thread builder;          // FSTX_CREATE_ASYNC: runs build_context() behind fstx_ctx_create's back
+    uint64_t create_t0 = 0;
+    uint64_t small_block = 0;     // block size for requests under kSmallRequest
+    uint32_t small_workers = 0;   // workers such a request wakes on an idle context
+    int64_t failed = 0;           // build failure, reported by every submit from then on (q_mutex)
 
     // fstx_ctx_order_after: one event, recorded on the caller's stream, awaited by the copy streams
     std::mutex order_mutex;
@@ -768,16 +783,21 @@ struct Worker {
         ctx->q_cv.notify_all();
     }
 
-    // the worker's share of the ring and the events that guard its slots
+    // the events that guard this worker's slots (the ring itself may not exist yet)
     int make_slots() {
         for (uint32_t k = 0; k < ctx->cfg.slots_per_thread; ++k) {
             Slot s;
-            s.host = ctx->ring + ((uint64_t)index * ctx->cfg.slots_per_thread + k) * ctx->slot_bytes;
             int rc = fstx_dev::event_create(&s.ev);
             if (rc < 0) return rc;
             mine->push_back(s);
         }
         return 0;
+    }
+
+    // the worker's share of the ring
+    void place_slots() {
+        for (uint32_t k = 0; k < mine->size(); ++k)
+            (*mine)[k].host = ctx->ring + ((uint64_t)index * ctx->cfg.slots_per_thread + k) * ctx->slot_bytes;
     }
 
     // Map the ring's pages into the process before the first block needs them: pinned memory
@@ -791,12 +811,13 @@ struct Worker {
     // queued: from then on the reads touch what is left as they go.
     void pretouch(uint32_t helpers) {
         const uint64_t slots = (uint64_t)ctx->cfg.n_threads * ctx->cfg.slots_per_thread;
-        const uint64_t head = std::min(ctx->slot_bytes, kSmallRequestBlock + kPage);
+        const uint64_t head = std::min(ctx->slot_bytes, ctx->small_block + kPage);
         uint64_t done = 0;
         char sink = 0;
         for (int pass = 0; pass < 2; ++pass) {
             const uint64_t from = pass == 0 ? 0 : head, to = pass == 0 ? head : ctx->slot_bytes;
             for (uint64_t s = index; s < slots; s += helpers) {
+                if (pass == 0 && ctx->head_mapped[s].load(std::memory_order_relaxed)) continue; // its owner has been there
                 const char *base = ctx->ring + s * ctx->slot_bytes;
                 for (uint64_t at = from; at < to; at += kPage) {
                     if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
@@ -808,6 +829,29 @@ struct Worker {
                 }
             }
         }
+        (void)sink;
+        ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
+    }
+
+    // The same for this worker's own slots, while the context is still being built: the part of
+    // each slot that the blocks of a small request use.  Stops once the streams exist and work
+    // is queued -- from then on a page is mapped when a read first writes to it.
+    void pretouch_own() {
+        const uint64_t head = std::min(ctx->slot_bytes, ctx->small_block + kPage);
+        uint64_t done = 0;
+        char sink = 0;
+        for (uint32_t k = 0; k < mine->size(); ++k) {
+            const char *base = (*mine)[k].host;
+            for (uint64_t at = 0; at < head; at += kPage) {
+                if ((at & (16 * kPage - 1)) == 0 && ctx->parts_seen.load(std::memory_order_acquire) &&
+                    ctx->work_seen.load(std::memory_order_acquire))
+                    goto out;
+                sink ^= *(const volatile char *)(base + at);
+                done += kPage;
+            }
+            ctx->head_mapped[(uint64_t)index * ctx->cfg.slots_per_thread + k].store(1, std::memory_order_relaxed);
+        }
+    out:
         (void)sink;
         ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
     }
@@ -827,13 +871,28 @@ struct Worker {
         mine = &ctx->slots[index];
         if (dev_rc == 0) dev_rc = make_slots();
         {
-            std::lock_guard<std::mutex> lk(ctx->ready_mutex);
+            // the ring is allocated by another thread meanwhile
+            std::unique_lock<std::mutex> lk(ctx->ready_mutex);
+            ctx->ready_cv.wait(lk, [&] { return ctx->ring_ready || ctx->parts_ready; });
+            if (dev_rc == 0 && !ctx->ring) dev_rc = ctx->parts_status ? ctx->parts_status : -FSTX_E_HIP;
+        }
+        if (dev_rc == 0) {
+            place_slots();
+            // until the streams exist there is nothing else to do: map what a small request will use
+            if (!ctx->no_read && !(ctx->cfg.flags & FSTX_NO_PRETOUCH) && index < ctx->small_workers) pretouch_own();
+        }
+        {
+            std::unique_lock<std::mutex> lk(ctx->ready_mutex);
+            ctx->ready_cv.wait(lk, [&] { return ctx->parts_ready; });
+            if (dev_rc == 0) dev_rc = ctx->parts_status;
+            if (dev_rc == 0) {
+                stream_ix = index % (uint32_t)ctx->streams.size();
+                stream = ctx->streams[stream_ix];
+            }
             ++ctx->ready;
             if (dev_rc < 0 && ctx->ready_status == 0) ctx->ready_status = (int)dev_rc;
         }
         ctx->ready_cv.notify_all();
-        stream_ix = index % (uint32_t)ctx->streams.size();
-        stream = ctx->streams[stream_ix];
         if (dev_rc == 0 && !ctx->no_read && !(ctx->cfg.flags & FSTX_NO_PRETOUCH)) {
             const uint32_t helpers = std::min(std::min(ctx->cfg.n_threads, 8u), std::max(1u, std::thread::hardware_concurrency() / 2));
             if (index < helpers) pretouch(helpers);
@@ -1061,7 +1120,7 @@ int normalize(fstx_config &cfg) {
     // max_direct_reads and direct_read_bytes stay 0 when the caller leaves them open: they are
     // settled from the block device under the first file that is opened for O_DIRECT
     if (cfg.block_bytes % kPage || cfg.n_threads > 1024 || cfg.n_streams > 64 || cfg.slots_per_thread > 64 ||
-        (cfg.flags & ~(FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_NO_COPY | FSTX_PROBE_NO_READ | FSTX_NO_PRETOUCH)))
+        (cfg.flags & ~(FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_NO_COPY | FSTX_PROBE_NO_READ | FSTX_NO_PRETOUCH | FSTX_CREATE_ASYNC)))
         return -FSTX_E_INVAL;
     if (cfg.direct_read_bytes)
         cfg.direct_read_bytes = std::max(cfg.block_bytes, align_down(cfg.direct_read_bytes, cfg.block_bytes));
@@ -1110,7 +1169,9 @@ std::vector<Shared> g_shared;
 bool same_config(const fstx_config &a, const fstx_config &b) {
     return a.device_id == b.device_id && a.numa_node == b.numa_node && a.n_threads == b.n_threads &&
            a.n_streams == b.n_streams && a.block_bytes == b.block_bytes && a.slots_per_thread == b.slots_per_thread &&
-           a.max_direct_reads == b.max_direct_reads && a.direct_read_bytes == b.direct_read_bytes && a.flags == b.flags &&
+           a.max_direct_reads == b.max_direct_reads && a.direct_read_bytes == b.direct_read_bytes &&
+           // how the context came to be is not part of what it is
+           (a.flags & ~FSTX_CREATE_ASYNC) == (b.flags & ~FSTX_CREATE_ASYNC) &&
            a.direct_ramp_kb == b.direct_ramp_kb;
 }
 
@@ -1161,6 +1222,140 @@ void settle_direct_shape(fstx_ctx *ctx, const StorageFacts &facts) {
 
 } // namespace
 
+namespace {
+
+// Ring, streams, events and workers of a context whose configuration has been checked.
+// The workers start first and make their events while a thread of its own allocates the ring
+// (bound to the node, so that the ring is placed there and the caller's affinity and memory
+// policy stay as they are; one allocation: sixteen small ones take ten times as long) and
+// this thread creates the streams: the build takes as long as its slowest part.  Returns 0 or
+// the first failure; the workers exist and run either way (after a failure they count off
+// every block with that status), so that tearing down is the same in both cases.
+int build_context(fstx_ctx *ctx) {
+    const fstx_config &cfg = ctx->cfg;
+    void *p = nullptr;
+    int ring_rc = 0, bound = 0, ring_node = -1;
+    uint64_t t_ring = 0;
+    std::thread placer([&] {
+        bound = bind_thread_to_node(cfg.numa_node);
+        ring_rc = fstx_dev::set_device(cfg.device_id);
+        if (ring_rc == 0) ring_rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
+        if (ring_rc == 0 && p && cfg.numa_node >= 0) {
+            *static_cast<volatile char *>(p) = 0; // the page exists from here on, on the node the policy names
+            ring_node = node_of_address(p);
+        }
+        t_ring = now_ns();
+        {
+            // the workers take their slots and begin to map them while the streams are still being made
+            std::lock_guard<std::mutex> lk(ctx->ready_mutex);
+            if (p) {
+                ctx->ring = static_cast<char *>(p);
+                fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
+            } else {
+                ctx->parts_status = ring_rc ? ring_rc : -FSTX_E_HIP;
+            }
+            ctx->ring_node = ring_node;
+            ctx->ring_ready = true;
+        }
+        ctx->ready_cv.notify_all();
+    });
+    int spawn_rc = 0;
+    try {
+        for (uint32_t t = 0; t < cfg.n_threads; ++t) {
+            ctx->workers.emplace_back([ctx, t] {
+                Worker w{ctx, t};
+                w.run();
+            });
+        }
+    } catch (const std::system_error &) {
+        spawn_rc = -EAGAIN;
+    }
+    const uint64_t t_spawned = now_ns();
+    int rc = fstx_dev::set_device(cfg.device_id);
+    for (uint32_t i = 0; i < cfg.n_streams && rc == 0; ++i) {
+        fstx_dev::stream_t s = nullptr;
+        if ((rc = fstx_dev::stream_create(&s)) == 0) ctx->streams.push_back(s);
+    }
+    if (rc == 0) rc = fstx_dev::event_create(&ctx->order_event);
+    const uint64_t t_streams = now_ns();
+    placer.join();
+    if (rc == 0) rc = ring_rc;
+    if (rc == 0) rc = spawn_rc;
+    if (bound < 0) {
+        ctx->ctr.bind_errors.fetch_add(1);
+        int64_t none = 0;
+        ctx->ctr.first_bind_error.compare_exchange_strong(none, bound);
+    }
+    {
+        std::unique_lock<std::mutex> lk(ctx->ready_mutex);
+        ctx->parts_status = rc;
+        ctx->parts_ready = true;
+        ctx->parts_seen.store(true, std::memory_order_release);
+        ctx->ready_cv.notify_all();
+        // a context exists once every worker has its slots
+        const uint32_t started = (uint32_t)ctx->workers.size();
+        ctx->ready_cv.wait(lk, [&] { return ctx->ready == started; });
+        if (rc == 0) rc = ctx->ready_status;
+    }
+    if (rc < 0) {
+        // submits fail from here on; what is queued already is counted off by the workers, and by
+        // this thread when not one of them could be started
+        std::deque<Block> orphans;
+        {
+            std::lock_guard<std::mutex> lk(ctx->q_mutex);
+            ctx->failed = rc;
+            if (ctx->workers.empty()) {
+                orphans.swap(ctx->queue);
+                ctx->queue_bytes = 0;
+            }
+        }
+        for (Block &b : orphans) {
+            int64_t none = 0;
+            b.req->error.compare_exchange_strong(none, rc);
+            if (b.req->blocks_left.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+                std::lock_guard<std::mutex> lk(ctx->done_mutex);
+                ctx->done_cv.notify_all();
+            }
+        }
+    }
+    ctx->create_ns = now_ns() - ctx->create_t0;
+    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu in %.2f ms (workers started %.2f, streams %.2f, ring %.2f)%s; "
+                         "node %d: %llu of %u workers on it, ring on node %d, %llu failed bindings (first: %lld); status %d",
+                         cfg.device_id, cfg.n_threads, cfg.n_streams, (unsigned long long)cfg.block_bytes,
+                         (unsigned long long)ctx->ring_bytes, ctx->create_ns / 1e6, (t_spawned - ctx->create_t0) / 1e6,
+                         (t_streams - ctx->create_t0) / 1e6, (t_ring - ctx->create_t0) / 1e6,
+                         (cfg.flags & FSTX_CREATE_ASYNC) ? ", behind the caller's back" : "", cfg.numa_node,
+                         (unsigned long long)ctx->ctr.workers_on_node.load(), cfg.n_threads, ctx->ring_node,
+                         (unsigned long long)ctx->ctr.bind_errors.load(), (long long)ctx->ctr.first_bind_error.load(), rc);
+    {
+        std::lock_guard<std::mutex> lk(ctx->ready_mutex);
+        ctx->build_status = rc;
+        ctx->built = true;
+    }
+    ctx->ready_cv.notify_all();
+    return rc;
+}
+
+// the build's status, once it is over (at once for a context that was built by its creator)
+int wait_built(fstx_ctx *ctx) {
+    std::unique_lock<std::mutex> lk(ctx->ready_mutex);
+    ctx->ready_cv.wait(lk, [&] { return ctx->built; });
+    return ctx->build_status;
+}
+
+void teardown(fstx_ctx *ctx) {
+    if (ctx->builder.joinable()) ctx->builder.join();
+    stop_workers(ctx);
+    fstx_dev::set_device(ctx->cfg.device_id);
+    for (auto s : ctx->streams) fstx_dev::stream_sync(s);
+    for (auto &kv : ctx->files) release_file(*kv.second);
+    for (char *p : ctx->stage_free) std::free(p);
+    free_parts(ctx);
+    delete ctx;
+}
+
+} // namespace
+
 int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
     *out = nullptr;
@@ -1172,82 +1367,50 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     int n_dev = fstx_dev::device_count();
     if (n_dev < 0) return n_dev;
     if (cfg.device_id < 0 || cfg.device_id >= n_dev) return -FSTX_E_INVAL;
-    rc = fstx_dev::set_device(cfg.device_id);
-    if (rc < 0) return rc;
 
     std::unique_ptr<fstx_ctx> ctx(new fstx_ctx);
     ctx->cfg = cfg;
+    ctx->create_t0 = t_start;
     ctx->no_copy = (cfg.flags & FSTX_PROBE_NO_COPY) != 0;
     ctx->no_read = (cfg.flags & FSTX_PROBE_NO_READ) != 0;
     ctx->direct_gate.reset(new Gate(1, 1, false));
     // a configuration that names both depth and size needs no device to settle on
     if (cfg.max_direct_reads && cfg.direct_read_bytes) settle_direct_shape(ctx.get(), StorageFacts{});
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
+    ctx->small_block = kSmallRequestBlock;
+    if (const char *e = std::getenv("FSTX_SMALL_BLOCK_KB")) {
+        const uint64_t kb = std::strtoull(e, nullptr, 10);
+        if (kb >= 64 && kb % 4 == 0) ctx->small_block = kb * 1024;
+    }
 
+    ctx->small_workers = std::min(cfg.n_threads, std::max(4u, cfg.n_threads / 2));
+    if (const char *e = std::getenv("FSTX_SMALL_WORKERS")) {
+        const uint64_t n = std::strtoull(e, nullptr, 10);
+        if (n >= 1) ctx->small_workers = (uint32_t)std::min<uint64_t>(n, cfg.n_threads);
+    }
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
     ctx->slot_bytes = cfg.block_bytes + kPage;
     ctx->ring_bytes = ctx->slot_bytes * cfg.n_threads * cfg.slots_per_thread;
     ctx->slots.resize(cfg.n_threads);
-    {
-        // One allocation (sixteen small ones take ten times as long), made by a thread of its
-        // own that binds itself to the node first: the ring is placed there and the caller's
-        // affinity and memory policy stay as they are.
-        void *p = nullptr;
-        int bound = 0, ring_node = -1;
-        std::thread placer([&] {
-            bound = bind_thread_to_node(cfg.numa_node);
-            rc = fstx_dev::set_device(cfg.device_id);
-            if (rc == 0) rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
-            if (rc == 0 && p && cfg.numa_node >= 0) {
-                *static_cast<volatile char *>(p) = 0; // the page exists from here on, on the node the policy names
-                ring_node = node_of_address(p);
-            }
-        });
-        placer.join();
-        if (rc < 0) return rc;
-        if (bound < 0) {
-            ctx->ctr.bind_errors.fetch_add(1);
-            ctx->ctr.first_bind_error.store(bound);
-        }
-        ctx->ring_node = ring_node;
-        ctx->ring = static_cast<char *>(p);
-        fstx_internal::note_bounce_bytes((int64_t)ctx->ring_bytes);
-    }
-    for (uint32_t i = 0; i < cfg.n_streams && rc == 0; ++i) {
-        fstx_dev::stream_t s = nullptr;
-        if ((rc = fstx_dev::stream_create(&s)) == 0) ctx->streams.push_back(s);
-    }
-    if (rc == 0) rc = fstx_dev::event_create(&ctx->order_event);
-    if (rc < 0) {
-        free_parts(ctx.get());
-        return rc;
-    }
+    ctx->head_mapped.reset(new std::atomic<uint8_t>[(size_t)cfg.n_threads * cfg.slots_per_thread]);
+    for (uint64_t i = 0; i < (uint64_t)cfg.n_threads * cfg.slots_per_thread; ++i) ctx->head_mapped[i].store(0);
     fstx_ctx *raw = ctx.release();
-    for (uint32_t t = 0; t < cfg.n_threads; ++t) {
-        raw->workers.emplace_back([raw, t] {
-            Worker w{raw, t};
-            w.run();
-        });
+    if (cfg.flags & FSTX_CREATE_ASYNC) {
+        // the caller goes on (headers to parse, files to open, reads to queue); whatever needs the
+        // streams or the outcome of the build waits for it
+        try {
+            raw->builder = std::thread([raw] { build_context(raw); });
+            *out = raw;
+            return 0;
+        } catch (const std::system_error &) {
+            // no thread to be had: build it here
+        }
     }
-    {
-        // the workers allocate their shares of the ring; a context exists once all of them have
-        std::unique_lock<std::mutex> lk(raw->ready_mutex);
-        raw->ready_cv.wait(lk, [&] { return raw->ready == cfg.n_threads; });
-        rc = raw->ready_status;
-    }
+    rc = build_context(raw);
     if (rc < 0) {
-        stop_workers(raw);
-        free_parts(raw);
-        delete raw;
+        teardown(raw);
         return rc;
     }
-    raw->create_ns = now_ns() - t_start;
-    fstx_internal::debug("ctx_create: device=%d threads=%u streams=%u block=%llu ring=%llu in %.2f ms; node %d: %llu of %u workers on it, "
-                         "ring on node %d, %llu failed bindings (first: %lld)", cfg.device_id,
-                         cfg.n_threads, cfg.n_streams, (unsigned long long)cfg.block_bytes,
-                         (unsigned long long)raw->ring_bytes, raw->create_ns / 1e6, cfg.numa_node,
-                         (unsigned long long)raw->ctr.workers_on_node.load(), cfg.n_threads, raw->ring_node,
-                         (unsigned long long)raw->ctr.bind_errors.load(), (long long)raw->ctr.first_bind_error.load());
     *out = raw;
     return 0;
 }
@@ -1255,6 +1418,7 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 int fstx_ctx_destroy(fstx_ctx *ctx) {
     if (!ctx) return -FSTX_E_INVAL;
     const uint64_t t0 = now_ns();
+    if (ctx->builder.joinable()) ctx->builder.join();
     stop_workers(ctx);
     const uint64_t t1 = now_ns();
     if (ctx->adaptive_depth && ctx->ctr.blocks_direct.load() > 64) g_depth_hint.store(ctx->direct_gate->settled());
@@ -1313,6 +1477,7 @@ int fstx_ctx_order_after(fstx_ctx *ctx, void *stream) {
     // an idle stream can still complete late, when that stream shares a hardware queue with a
     // busy one.)
     if (fstx_dev::stream_idle(stream) == 1) return 0;
+    if ((rc = wait_built(ctx)) < 0) return rc; // the copy streams are needed from here on
     rc = fstx_dev::event_record(ctx->order_event, stream);
     for (size_t i = 0; i < ctx->streams.size() && rc == 0; ++i) rc = fstx_dev::stream_wait_event(ctx->streams[i], ctx->order_event);
     return rc;
@@ -1417,7 +1582,7 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
         // it uses has been touched once -- 2.5 ms for 32 slots of 2 MiB, which is a sixth of a
         // 0.7 GB load.  1 MiB blocks still run the link at 56 of its 57 GB/s.
         uint64_t bb = ctx->cfg.block_bytes;
-        if (length < kSmallRequest) bb = std::min(bb, kSmallRequestBlock);
+        if (length < kSmallRequest) bb = std::min(bb, ctx->small_block);
         const uint64_t origin = align_down(file_off, kPage);
         const uint64_t end = file_off + length;
         for (uint64_t lo = origin; lo < end; lo += bb) {
@@ -1429,15 +1594,15 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
     if (!blocks.empty()) {
         {
             std::lock_guard<std::mutex> lk(ctx->q_mutex);
-            if (ctx->closing) {
+            if (ctx->closing || ctx->failed) {
                 std::lock_guard<std::mutex> lk2(ctx->table_mutex);
                 ctx->requests.erase(req->id);
                 req->file->open_requests.fetch_sub(1);
-                return -FSTX_E_CLOSED;
+                return ctx->failed ? ctx->failed : -FSTX_E_CLOSED;
             }
             const bool idle = ctx->queue.empty() && ctx->staged.empty();
             const uint32_t all = ctx->cfg.n_threads;
-            ctx->active_workers = idle && length < kSmallRequest ? std::min(all, std::max(4u, all / 2)) : all;
+            ctx->active_workers = idle && length < kSmallRequest ? ctx->small_workers : all;
             for (Block &b : blocks) {
                 ctx->queue_bytes += b.len;
                 ctx->queue.push_back(std::move(b));
@@ -1477,6 +1642,10 @@ int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request) {
     // and waited for instead.
     int64_t status = req->error.load();
     const uint64_t mask = req->stream_mask.load();
+    if (mask == 0) { // nothing went to a stream: an empty request, a failed one, or a context that could not be built
+        req->file->open_requests.fetch_sub(1);
+        return status < 0 ? status : (int64_t)req->length;
+    }
     fstx_dev::set_device(ctx->cfg.device_id);
     if (alone) {
         for (size_t i = 0; i < ctx->streams.size(); ++i)
@@ -1528,6 +1697,7 @@ int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
     // the caller says how large its struct is; a caller built against an older header gets the
     // fields it knows and nothing is written behind them
     if (!ctx || !out || out->struct_size < 2 * sizeof(uint64_t)) return -FSTX_E_INVAL;
+    (void)wait_built(ctx); // where the workers and the ring ended up is part of the answer
     const Counters &c = ctx->ctr;
     fstx_metrics m{};
     m.struct_size = std::min<uint64_t>(out->struct_size, sizeof(fstx_metrics));

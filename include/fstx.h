@@ -77,7 +77,7 @@ typedef struct fstx_config {
                                    queue's worth (nr_requests x max_sectors_kb, 64 MiB .. 1 GiB)
                                    with one read in flight, a quarter of it with several, and
                                    never more staging memory than 1/16 of MemAvailable           */
-    uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_*                               */
+    uint32_t flags;          /* FSTX_ADAPTIVE_DEPTH | FSTX_PROBE_* | FSTX_NO_PRETOUCH | FSTX_CREATE_ASYNC */
     uint32_t direct_ramp_kb; /* KiB of the first O_DIRECT pread after the queue was empty; the next
                                 ones are 4x, 16x .. as large up to direct_read_bytes, and towards the
                                 end of the queued bytes they halve down to this size again, so that
@@ -101,6 +101,13 @@ typedef struct fstx_config {
 /* The workers do not map the pages of their ring slots ahead of the first request (they do by
  * default: pinned memory is mapped at its first touch, which is slow); for measurements. */
 #define FSTX_NO_PRETOUCH 8u
+/* fstx_ctx_create / fstx_ctx_acquire return as soon as the configuration has been checked; a
+ * thread of the library builds ring, streams and workers meanwhile (about a millisecond, during
+ * which the caller parses headers, opens files and queues reads: none of that waits).  The calls
+ * that need the outcome wait for it: fstx_wait_read, fstx_get_metrics, fstx_ctx_order_after on a
+ * busy stream, fstx_ctx_destroy.  A build that fails is reported by fstx_wait_read for whatever
+ * was queued, and by every fstx_submit_read after it. */
+#define FSTX_CREATE_ASYNC 16u
 
 /* fstx_metrics.storage_flags */
 #define FSTX_STORAGE_KNOWN 1u      /* the block layer named queue depth and request size          */
@@ -122,7 +129,8 @@ typedef struct fstx_metrics {
     uint64_t direct_depth;        /* O_DIRECT preads allowed in flight (steered: the depth last
                                      found good, not a step that is still being tried)           */
     uint64_t direct_reads;        /* O_DIRECT preads issued (each covers a run of blocks)        */
-    uint64_t create_ns;           /* what fstx_ctx_create took: threads, ring, streams, events   */
+    uint64_t create_ns;           /* from the call of fstx_ctx_create until threads, ring, streams
+                                     and events existed                                           */
     /* where the I/O side runs (fstx_config.numa_node >= 0) */
     int64_t numa_node;            /* the node asked for, -1 = none                               */
     uint64_t workers_on_node;     /* workers whose CPU affinity, read back with sched_getaffinity

@@ -92,6 +92,8 @@ StorageModel g_storage;
 std::atomic<int> g_copy_delay_us{50};
 std::atomic<int64_t> g_fail_copy_after{-1};
 std::atomic<int64_t> g_pinned_live{0};
+std::atomic<int> g_host_alloc_delay_us{0};
+std::atomic<int> g_host_alloc_failures{0};
 
 } // namespace
 
@@ -120,6 +122,9 @@ void fstx_test_after_direct_read(uint64_t bytes) {
     g_storage.cv.notify_one();
 }
 void fstx_sim_fail_copy_after(int64_t n) { g_fail_copy_after.store(n); }
+// the pinned allocation takes this long (a slow context build), and the next `n` of them fail
+void fstx_sim_set_host_alloc_delay_us(int us) { g_host_alloc_delay_us.store(us); }
+void fstx_sim_fail_host_allocs(int n) { g_host_alloc_failures.store(n); }
 int64_t fstx_sim_pinned_live(void) { return g_pinned_live.load(); }
 // a caller-side stream: created here, handed to fstx_ctx_order_after as its `stream`
 void *fstx_sim_stream_create(void) { return new SimStream; }
@@ -142,6 +147,8 @@ int pci_bus_id(int, char *out, int len) {
     return 0;
 }
 int host_alloc(void **out, size_t bytes) {
+    if (int us = g_host_alloc_delay_us.load()) std::this_thread::sleep_for(std::chrono::microseconds(us));
+    if (g_host_alloc_failures.load() > 0 && g_host_alloc_failures.fetch_sub(1) > 0) return -FSTX_E_HIP;
     if (posix_memalign(out, 4096, bytes ? bytes : 1) != 0) return -FSTX_E_HIP;
     g_pinned_live.fetch_add(1);
     return 0;

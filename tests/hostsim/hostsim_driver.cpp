@@ -55,7 +55,8 @@ int main(int argc, char **argv) {
         cfg.block_bytes = 4096u << (round * 2);
         cfg.slots_per_thread = 1 + round % 2;
         cfg.direct_read_bytes = round == 1 ? 0 : cfg.block_bytes * 3;
-        cfg.flags = round == 2 ? FSTX_ADAPTIVE_DEPTH : 0;
+        // rounds 0 and 1: the context is built behind the callers' backs while they open files and queue reads
+        cfg.flags = round == 2 ? FSTX_ADAPTIVE_DEPTH : FSTX_CREATE_ASYNC;
         cfg.direct_ramp_kb = round == 0 ? 4 : 0;
         fstx_ctx *ctx = nullptr, *again = nullptr;
         // odd rounds go through the shared table: two users of one context

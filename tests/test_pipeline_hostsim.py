@@ -38,6 +38,8 @@ def sim():
     lib.fstx_sim_stream_create.restype = ctypes.c_void_p
     lib.fstx_sim_stream_destroy.argtypes = [ctypes.c_void_p]
     lib.fstx_sim_stream_sleep_then_set.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
+    lib.fstx_sim_set_host_alloc_delay_us.argtypes = [ctypes.c_int]
+    lib.fstx_sim_fail_host_allocs.argtypes = [ctypes.c_int]
     lib.fstx_sim_set_copy_delay_us(30)
     return lib
 
@@ -165,6 +167,77 @@ def test_error_paths(sim, blob, tmp_path):
 def _native_code(name: str) -> int:
     return {"INVAL": 10001, "HIP": 10002, "RANGE": 10003, "SHORT_READ": 10004, "NO_REQ": 10005,
             "CLOSED": 10006, "NO_DEVICE": 10007, "TOO_MANY": 10008}[name]
+
+
+def test_context_built_behind_the_callers_back(sim, blob):
+    """FSTX_CREATE_ASYNC: create returns before ring, streams and workers exist (here the pinned
+    allocation takes 150 ms); files are opened and reads queued meanwhile, and the wait delivers
+    the bytes once the build is through.  The same configuration without the flag names the same
+    shared context."""
+    path, data = blob
+    import time
+
+    sim.fstx_sim_set_host_alloc_delay_us(150_000)
+    try:
+        t0 = time.perf_counter()
+        ctx = make_ctx(sim, block=64 * 1024, flags=_native.CREATE_ASYNC)
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        dev = np.zeros(data.size, dtype=np.uint8)
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        queued_after = time.perf_counter() - t0
+        assert req >= 1 and queued_after < 0.1, queued_after  # nothing waited for the build
+        assert sim.fstx_wait_read(ctx, req) == data.size
+        assert time.perf_counter() - t0 >= 0.15
+        assert np.array_equal(dev, data)
+        m = metrics(sim, ctx)
+        assert m.create_ns >= 150_000_000 and m.bytes_copied == data.size
+        assert sim.fstx_file_close(ctx, f) == 0
+        # destroying a context right after asking for it waits for the build, then takes it apart
+        other = make_ctx(sim, block=8192, flags=_native.CREATE_ASYNC)
+        assert sim.fstx_ctx_destroy(other) == 0
+        assert sim.fstx_ctx_destroy(ctx) == 0
+        assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+    finally:
+        sim.fstx_sim_set_host_alloc_delay_us(0)
+    a = make_ctx(sim, block=16384, flags=_native.CREATE_ASYNC, shared=True)
+    b = make_ctx(sim, block=16384, flags=0, shared=True)
+    assert a.value == b.value
+    assert sim.fstx_ctx_release(a) == 0 and sim.fstx_ctx_release(b) == 0
+    assert sim.fstx_bounce_buffer_bytes() == 0
+
+
+def test_a_failed_build_is_reported_by_whoever_waits(sim, blob):
+    """The pinned allocation fails.  Built by the creator, fstx_ctx_create returns the error and
+    leaves nothing behind; built behind the caller's back, the reads that were queued meanwhile
+    fail at their wait, later submits are refused with the same status, and destroy cleans up."""
+    path, data = blob
+    out = ctypes.c_void_p()
+    cfg = make_cfg(block=64 * 1024)
+    sim.fstx_sim_fail_host_allocs(1)
+    assert sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(out)) == -_native_code("HIP")
+    assert not out.value and sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+    sim.fstx_sim_set_host_alloc_delay_us(50_000)
+    sim.fstx_sim_fail_host_allocs(1)
+    try:
+        ctx = make_ctx(sim, block=64 * 1024, flags=_native.CREATE_ASYNC)
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        dev = np.zeros(data.size, dtype=np.uint8)
+        reqs = [sim.fstx_submit_read(ctx, f, at, 1 << 20, dev.ctypes.data, dev.size, at) for at in (0, 1 << 20, 2 << 20)]
+        assert all(r >= 1 for r in reqs)
+        assert [sim.fstx_wait_read(ctx, r) for r in reqs] == [-_native_code("HIP")] * 3
+        assert not dev.any()
+        assert sim.fstx_submit_read(ctx, f, 0, 4096, dev.ctypes.data, dev.size, 0) == -_native_code("HIP")
+        stream = sim.fstx_sim_stream_create()
+        flag = ctypes.c_int(0)
+        sim.fstx_sim_stream_sleep_then_set(stream, 20_000, ctypes.byref(flag), 1)
+        assert sim.fstx_ctx_order_after(ctx, stream) == -_native_code("HIP")
+        sim.fstx_sim_stream_destroy(stream)
+        assert sim.fstx_file_close(ctx, f) == 0
+        assert sim.fstx_ctx_destroy(ctx) == 0
+        assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+    finally:
+        sim.fstx_sim_set_host_alloc_delay_us(0)
+        sim.fstx_sim_fail_host_allocs(0)
 
 
 def test_injected_read_fault(sim, blob):
