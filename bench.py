@@ -727,6 +727,78 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         del ts, outs
     out["join_odd_columns"] = odd_joins
 
+    # -- short segments: tiles that hold many of them (every lane finds its own segment), a narrow
+    #    block written into a wide tensor, and the small-unit fallback for segments under 16 bytes
+    short = {}
+
+    def row(label, kernel, nb, launch, check, torch_way=None):
+        launch()
+        ms = timed([launch] * 5)
+        if not check():
+            raise SystemExit(f"bench: {label}: result differs from torch's slicing")
+        short[label] = {"kernel": kernel, "avg_launch_ms": sum(ms) / len(ms), "bytes_per_launch": nb,
+                        "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
+        if torch_way is not None:
+            # the same bytes moved by torch's own strided copy, for scale (one pair of events around the whole of it)
+            torch_way()
+            tm = timed([torch_way] * 3)
+            short[label]["torch_strided_copy_GBps"] = nb / 1e6 / (sum(tm) / len(tm))
+
+    rows_n, width, count = 88064, 1016, 24
+    ts = [torch.randint(0, 255, (rows_n, width), dtype=torch.uint8, device=dev) for _ in range(count)]
+    blk = width // world
+    outs = [torch.empty((rows_n, count * blk), dtype=torch.uint8, device=dev) for _ in range(world)]
+    jsrc = [[(t.data_ptr() + r * blk, blk, width) for t in ts] for r in range(world)]
+    for r in range(world):
+        _native.join_copy(outs[r].data_ptr(), rows_n, jsrc[r], stream)
+    ms = timed([lambda r=r: _native.join_copy(outs[r].data_ptr(), rows_n, jsrc[r], stream) for r in range(world)] * 3)
+    for r in range(world):
+        if not torch.equal(outs[r], torch.cat([t[:, r * blk : (r + 1) * blk] for t in ts], dim=1)):
+            raise SystemExit("bench: join of short segments differs from slicing + cat")
+    nb = 2 * outs[0].numel()
+    short[f"{count} x u8 [{rows_n}, {width}], column blocks of a rank ({blk}-byte segments) joined along dim 1"] = {
+        "kernel": "gather_kernel<multi, keep>", "avg_launch_ms": sum(ms) / len(ms), "bytes_per_launch": nb,
+        "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
+    del outs, jsrc
+    t = ts[0]
+    del ts
+    big = torch.randint(0, 255, (1 << 20, width), dtype=torch.uint8, device=dev)
+    dsts = [torch.empty((big.shape[0], blk), dtype=torch.uint8, device=dev) for _ in range(world)]
+    jobs = [(dsts[r].data_ptr(), big.data_ptr() + r * blk, big.shape[0], blk, width) for r in range(world)]
+    row(f"u8 [{big.shape[0]}, {width}] cut in 4 along dim 1 ({blk}-byte segments), 4 ranks per launch", "gather_kernel<keep>",
+        2 * sum(d.numel() for d in dsts), lambda: _native.slice_copy_batch(jobs, stream),
+        lambda: all(torch.equal(dsts[r], big[:, r * blk : (r + 1) * blk]) for r in range(world)),
+        lambda: [dsts[r].copy_(big[:, r * blk : (r + 1) * blk]) for r in range(world)])
+    del dsts
+    # a rank's narrow column block written into its columns of a wide tensor: through the gather kernel
+    # (vectors counted row by row from each row's own first byte) and, for scale, through the unit kernel
+    for seg, pitch, dpitch, n_rows in [(96, 384, 4096, 1 << 20), (94, 377, 4094, 1 << 20), (1024, 4096, 8192, 1 << 18),
+                                       (1000, 4000, 8000, 1 << 18)]:
+        src = torch.randint(0, 255, (n_rows, pitch), dtype=torch.uint8, device=dev)
+        wide = torch.zeros((n_rows, dpitch), dtype=torch.uint8, device=dev)
+        job = [(wide.data_ptr() + 128, src.data_ptr() + seg, n_rows, seg, pitch, dpitch)]
+        label = f"[{n_rows}, {seg}]-byte block (pitch {pitch}) into columns 128.. of a tensor with {dpitch}-byte rows"
+        row(label, "gather_kernel<pitched>, vectors counted row by row", 2 * n_rows * seg, lambda: _native.slice_copy2d_batch(job, stream),
+            lambda: torch.equal(wide[:, 128 : 128 + seg], src[:, seg : 2 * seg]) and not wide[:, :128].any() and not wide[:, 128 + seg :].any(),
+            lambda: wide[:, 128 : 128 + seg].copy_(src[:, seg : 2 * seg]))
+        os.environ["FSTX_GATHER_MODE"] = "0"
+        _native.slice_copy2d_batch(job, stream)
+        ms = timed([lambda: _native.slice_copy2d_batch(job, stream)] * 5)
+        os.environ.pop("FSTX_GATHER_MODE")
+        short[label]["slice2d_kernel_GBps"] = 2 * n_rows * seg / 1e6 / (sum(ms) / len(ms))
+        del src, wide
+    # segments under 16 bytes: bf16 [N, 4] cut in 4 along dim 1, one 2-byte element per row and rank
+    thin = torch.randint(-32768, 32767, (1 << 25, 4), dtype=torch.int16, device=dev)
+    douts = [torch.empty((thin.shape[0], 1), dtype=torch.int16, device=dev) for _ in range(world)]
+    jobs2 = [(douts[r].data_ptr(), thin.data_ptr() + 2 * r, thin.shape[0], 2, 8) for r in range(world)]
+    row(f"bf16 [{thin.shape[0]}, 4] cut in 4 along dim 1 (2-byte segments), 4 ranks per launch", "slice2d_kernel, 2-byte units",
+        2 * sum(d.numel() * 2 for d in douts), lambda: _native.slice_copy_batch(jobs2, stream),
+        lambda: all(torch.equal(douts[r], thin[:, r : r + 1]) for r in range(world)),
+        lambda: [douts[r].copy_(thin[:, r : r + 1]) for r in range(world)])
+    del thin, douts, big, t
+    out["short_segments"] = short
+    torch.cuda.empty_cache()
+
     # -- realign: config C2's data section shifted by header_length % 16 = 10 bytes
     n = 709_646_336
     cal = 1 << 30

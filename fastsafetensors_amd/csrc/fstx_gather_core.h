@@ -60,12 +60,15 @@ struct alignas(64) Job {
     const char *src;    // nsrc == 1: first byte of the block in row 0
     uint64_t pitch;     // nsrc == 1: bytes between its rows; nsrc > 1: magic_of(equal_seg), or 0
     uint32_t seg;       // nsrc == 1: bytes per row, >= kMinSeg
-    uint32_t flags;     // kByRows
-    uint64_t pitch_magic; // magic_of(dst_pitch); kByRows: magic_of(vectors_per_row(row_bytes))
+    uint32_t flags;     // kByRows | kShort | kLooseRows
+    uint64_t pitch_magic; // magic_of(dst_pitch); kByRows: magic_of(vectors per row)
 };
 
 // Job::flags
 constexpr uint32_t kByRows = 2; // vectors are counted row by row (see vectors_per_row)
+constexpr uint32_t kShort = 4;  // some segment is shorter than kShortSeg: a tile may hold more than three
+constexpr uint32_t kLooseRows = 8; // with kByRows, one source: a row's vectors begin at the row's own first byte
+constexpr uint32_t kShortSeg = 512;
 
 struct alignas(32) Src {
     const char *src; // first byte of the block in row 0
@@ -184,13 +187,23 @@ FSTX_HD Src src_uniform(const Src *more, uint32_t index) {
 #endif
 }
 
+// the column of table entry `index` alone (uniform index: one scalar dword)
+FSTX_HD uint32_t col_uniform(const Src *more, uint32_t index) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *reinterpret_cast<const uint32_t *>(
+        reinterpret_cast<const char *>(&more[__builtin_amdgcn_readfirstlane(index)]) + __builtin_offsetof(Src, col));
+#else
+    return more[index].col;
+#endif
+}
+
 // which source holds column c of a row (c < row_bytes): the table is read with scalar loads,
 // the comparisons are per lane
 FSTX_HD uint32_t source_of(const Job &jb, const Src *more, uint32_t c) {
     if (jb.nsrc == 1) return 0;
     if (jb.equal_seg) return div_magic(c, jb.pitch);
     uint32_t k = 0;
-    for (uint32_t i = 1; i < jb.nsrc; ++i) k += c >= src_uniform(more, jb.more0 + i).col ? 1u : 0u;
+    for (uint32_t i = 1; i < jb.nsrc; ++i) k += c >= col_uniform(more, jb.more0 + i) ? 1u : 0u;
     return k;
 }
 
@@ -219,9 +232,57 @@ FSTX_HD Piece piece_of(const Job &jb, const Src *more, uint32_t row, uint32_t c,
 // payload, vectors_per_row of them at most, and a vector never holds bytes of two rows (the gap
 // is at least a vector wide).
 FSTX_HD uint32_t vectors_per_row(uint32_t row_bytes) { return (row_bytes + 2 * (kVec - 1)) / kVec; }
+// One source: the vectors of a row are counted from the row's own first byte instead -- sixteen
+// bytes at dst_row + 16 v, wherever that is, and a last one that ends with the row (it overlaps
+// its neighbour when the row is not a multiple of sixteen bytes and writes the same bytes again).
+// Every vector is whole payload: one load and one store of sixteen bytes at their own addresses,
+// no partial vector and no byte-wise store anywhere in the job.
+FSTX_HD uint32_t loose_vectors_per_row(uint32_t row_bytes) { return (row_bytes + kVec - 1) / kVec; }
 inline bool counts_by_rows(uint64_t dst_pitch, uint64_t row_bytes) {
     const uint64_t gap = dst_pitch - row_bytes;
     return gap >= kVec && gap > dst_pitch / 8;
+}
+
+// Tiles of short segments (Job::flags & kShort: some segment is under kShortSeg bytes, so a tile
+// may hold four of them, or sixty).  No description of the tile is shared: every lane finds row,
+// source and offset of its own vector by arithmetic -- two multiply-highs, or a count over the
+// sources' columns when their widths differ -- fetches the two table entries it may need (its
+// segment's and the following one's) together, then issues its one or two data loads together:
+// two waits per wavefront, whatever the number of seams.  Decided once per wavefront: not the
+// job's first or last tile (the caller checks), and no lane of the tile in the first row or
+// beyond the last but one of its source block, so that a load which reaches up to 15 bytes
+// before or behind its segment stays inside the block.  Returns false for a tile, or on a
+// pitched destination a lane, that needs the general way.
+template <bool kMulti, bool kPitched, class Mem>
+FSTX_HD bool gather_lane_short(const Job &jb, const Src *more, uint32_t t_lo, uint32_t lane, Mem &mem) {
+    const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
+    const uint32_t row_first = div_magic(t_lo, jb.pitch_magic), row_last = div_magic(t_lo + kTile - 1, jb.pitch_magic);
+    if (row_first == 0 || row_last + 2 > jb.rows) return false;
+    const uint32_t q = t_lo + kVec * lane; // position of the vector's byte 0
+    const uint32_t row = div_magic(q, jb.pitch_magic);
+    const uint32_t c = q - row * dst_pitch;
+    if (kPitched && c >= jb.row_bytes) return false; // in the gap behind a row's payload
+    const bool multi = kMulti && jb.nsrc > 1;
+    Src s1 = {jb.src, jb.pitch, jb.seg, 0, 0}, s2 = s1;
+    uint32_t row2 = row + 1;
+    if (multi) {
+        const uint32_t k = source_of(jb, more, c);
+        const uint32_t k2 = k + 1 < jb.nsrc ? k + 1 : 0u;
+        // both entries before either is used
+        s1 = mem.table(more, jb.more0 + k);
+        s2 = mem.table(more, jb.more0 + k2);
+        row2 = k2 ? row : row + 1;
+    }
+    const uint32_t in1 = c - s1.col;
+    const uint32_t rest = s1.seg - in1;   // bytes of the segment from the vector's byte 0 on
+    const bool has2 = rest < kVec;        // it ends inside the vector: the following segment begins `rest` bytes in
+    if (kPitched && has2 && row2 != row) return false; // continues behind the gap: partly payload
+    Vec16 g2 = {{0, 0, 0, 0}};
+    const Vec16 g1 = mem.load16_stream(s1.src + (uint64_t)row * s1.pitch + in1);
+    if (has2) g2 = mem.load16(s2.src + (uint64_t)row2 * s2.pitch - rest);
+    const uint32_t from2 = has2 ? rest : kVec;
+    mem.store16(jb.dst + q, blend(g1, g2, from2, kVec - from2));
+    return true;
 }
 
 // The common tile, decided once per wavefront: not the job's first or last tile, at most three
@@ -242,6 +303,15 @@ FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, ui
         // inside that row's segment and one store (pitch_magic divides by the vectors per row here)
         if (kMulti && jb.nsrc > 1) return false;
         const uint32_t j = tile * kLanes + lane;
+        if (jb.flags & kLooseRows) {
+            if (j >= jb.nvec) return true;
+            const uint32_t per = loose_vectors_per_row(jb.row_bytes);
+            const uint32_t r = per == 1 ? j : div_magic(j, jb.pitch_magic);
+            const uint32_t at = kVec * (j - r * per);
+            const uint32_t off = at + kVec <= jb.row_bytes ? at : jb.row_bytes - kVec; // the last one ends with the row
+            mem.store16_any(jb.dst + (uint64_t)r * jb.dst_pitch + off, mem.load16_stream(jb.src + (uint64_t)r * jb.pitch + off));
+            return true;
+        }
         if (j >= jb.nvec) return false;
         const uint32_t per_row = vectors_per_row(jb.row_bytes);
         const uint32_t row = div_magic(j, jb.pitch_magic);
@@ -258,6 +328,7 @@ FSTX_HD bool gather_lane_inner(const Job &jb, const Src *more, uint32_t tile, ui
     const uint32_t head = (uint32_t)((uintptr_t)jb.dst & (kVec - 1));
     const uint32_t dst_pitch = kPitched ? jb.dst_pitch : jb.row_bytes;
     const uint32_t t_lo = tile * kTile - head; // position of the tile's first byte
+    if (jb.flags & kShort) return gather_lane_short<kMulti, kPitched>(jb, more, t_lo, lane, mem);
     uint32_t row = div_magic(t_lo, jb.pitch_magic);
     uint32_t c0 = t_lo - row * dst_pitch;
     if (kPitched && c0 >= jb.row_bytes) { // the tile begins in the gap behind a row's payload
@@ -466,16 +537,17 @@ inline uint64_t rows_per_job(uint64_t dst_pitch, uint64_t row_bytes) {
 // One source: `one` is it and more0 is unused.  Several: they sit at table[more0 .. more0 + nsrc)
 // of the launch and `one` is ignored.
 inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t rows, const Src &one, uint32_t more0,
-                    uint32_t nsrc, uint64_t equal_seg) {
+                    uint32_t nsrc, uint64_t equal_seg, uint64_t min_seg) {
     const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
     const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
-    const bool single = nsrc == 1, by_rows = counts_by_rows(dst_pitch, row_bytes);
-    const uint64_t nvec = by_rows ? rows * vectors_per_row((uint32_t)row_bytes) : (head + span + kVec - 1) / kVec;
+    const bool single = nsrc == 1, by_rows = counts_by_rows(dst_pitch, row_bytes), loose = by_rows && single;
+    const uint32_t per_row = loose ? loose_vectors_per_row((uint32_t)row_bytes) : vectors_per_row((uint32_t)row_bytes);
+    const uint64_t nvec = by_rows ? rows * per_row : (head + span + kVec - 1) / kVec;
     return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,
                (uint32_t)nvec, (uint32_t)(single ? 0 : equal_seg), single ? one.src : nullptr,
                single ? one.pitch : magic_of(equal_seg), single ? one.seg : 0u,
-               by_rows ? kByRows : 0u,
-               magic_of(by_rows ? vectors_per_row((uint32_t)row_bytes) : dst_pitch)};
+               (by_rows ? kByRows : 0u) | (loose ? kLooseRows : 0u) | (min_seg < kShortSeg ? kShort : 0u),
+               magic_of(by_rows ? per_row : dst_pitch)};
 }
 
 inline uint64_t tiles_of(const Job &jb) { return ((uint64_t)jb.nvec + kLanes - 1) / kLanes; }

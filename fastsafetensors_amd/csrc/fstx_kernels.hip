@@ -243,24 +243,69 @@ __device__ __forceinline__ void slice_units(const SliceJob &job, uint32_t u) {
     st_stream(ld_stream(src), dst);
 }
 
+// Units under 16 bytes into a 16-byte-aligned dense destination: a lane gathers the 16 / sizeof(Unit)
+// units of one destination vector -- as many loads, issued together -- and writes them with one
+// 16-byte store, so a wavefront still writes 1 KiB of contiguous memory (one unit per lane is
+// 64 to 512 bytes per wavefront).  `g` is the index of the destination vector.
+template <typename Unit>
+__device__ __forceinline__ void slice_units_packed(const SliceJob &job, uint32_t g) {
+    constexpr uint32_t kPer = kVecBytes / sizeof(Unit);
+    const uint32_t u0 = g * kPer; // < total_units + kPer, which the host keeps below 2^32
+    if (u0 >= job.total_units) return;
+    const uint64_t pitch = job.pitch_unit & 0x00ffffffffffffffull;
+    uint32_t row = u0 / job.seg_units;
+    uint32_t col = u0 - row * job.seg_units;
+    const uint32_t live = job.total_units - u0 < kPer ? job.total_units - u0 : kPer;
+    Unit part[kPer];
+#pragma unroll
+    for (uint32_t k = 0; k < kPer; ++k) {
+        part[k] = Unit{};
+        if (k < live) part[k] = ld_global(reinterpret_cast<const Unit *>(job.src + (uint64_t)row * pitch) + col);
+        if (++col == job.seg_units) {
+            col = 0;
+            ++row;
+        }
+    }
+    Unit *dst = reinterpret_cast<Unit *>(job.dst) + u0;
+    if (live == kPer) {
+        v4u whole;
+        __builtin_memcpy(&whole, part, sizeof whole);
+        st_stream(whole, reinterpret_cast<v4u *>(dst));
+    } else {
+#pragma unroll
+        for (uint32_t k = 0; k < kPer; ++k)
+            if (k < live) st_global(part[k], dst + k);
+    }
+}
+
+constexpr uint32_t kPackedUnits = 0x80; // in the unit byte of SliceJob::pitch_unit: slice_units_packed
+
 __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_log2,
                                                         const JobTable<SliceJob> t) {
     const uint32_t b = blockIdx.x;
     const uint32_t ji = find_job(t, granule_log2, b);
     const SliceJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
+    const uint32_t mode = (uint32_t)(job.pitch_unit >> 56);
+    // items: units, or (packed) destination vectors of 16 >> unit_log2 units
+    const uint32_t per_log2 = mode & kPackedUnits ? 4 - (mode & 7) : 0;
+    const uint32_t items = (uint32_t)(((uint64_t)job.total_units + (1u << per_log2) - 1) >> per_log2);
     // neighbouring workgroups on the same die, in the tile order of tile_for_die
     uint32_t tile;
-    if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
+    if (!tile_for_die(lb, (items + kBlock - 1) / kBlock, tile)) return;
     const uint64_t u64 = (uint64_t)tile * kBlock + threadIdx.x;
-    if (u64 >= job.total_units) return; // also retires the idle workgroups of a job's last granule
+    if (u64 >= items) return; // also retires the idle workgroups of a job's last granule
     const uint32_t u = (uint32_t)u64;
-    switch ((uint32_t)(job.pitch_unit >> 56)) { // uniform across the workgroup
+    switch (mode) { // uniform across the workgroup
     case 4: slice_units<v4u>(job, u); break;
     case 3: slice_units<uint64_t>(job, u); break;
     case 2: slice_units<uint32_t>(job, u); break;
     case 1: slice_units<uint16_t>(job, u); break;
-    default: slice_units<uint8_t>(job, u); break;
+    case 0: slice_units<uint8_t>(job, u); break;
+    case kPackedUnits | 3: slice_units_packed<uint64_t>(job, u); break;
+    case kPackedUnits | 2: slice_units_packed<uint32_t>(job, u); break;
+    case kPackedUnits | 1: slice_units_packed<uint16_t>(job, u); break;
+    default: slice_units_packed<uint8_t>(job, u); break;
     }
 }
 
@@ -317,8 +362,18 @@ typedef v4u v4u_anywhere __attribute__((aligned(1)));
 // parts of several segments, which neighbouring lanes and tiles fetch one after the other, and
 // the bulk loads are plain ones that leave the line in the caches (+14 % on a join of 254-byte
 // segments; on segments of 2 KB and more streaming loads are 1-5 % faster).
-constexpr uint64_t kShortSeg = 512;
+constexpr uint64_t kShortSeg = fstx_gather::kShortSeg;
 template <bool kKeep> struct GatherMem {
+    // one entry of the launch's source table, for a lane of its own (the table sits in the kernel
+    // arguments; two 16-byte loads that hit the same few lines in every wavefront)
+    __device__ __forceinline__ fstx_gather::Src table(const fstx_gather::Src *more, uint32_t index) {
+        const v4u a = *(const FSTX_GLOBAL v4u *)(&more[index]);
+        const v4u b = *((const FSTX_GLOBAL v4u *)(&more[index]) + 1);
+        fstx_gather::Src out;
+        const uint32_t raw[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        __builtin_memcpy(&out, raw, sizeof out);
+        return out;
+    }
     // the bulk: streaming loads (every byte of a checkpoint is cut once)
     __device__ __forceinline__ fstx_gather::Vec16 load16_stream(const char *p) {
         const v4u v = kKeep ? *(const FSTX_GLOBAL v4u_anywhere *)p : __builtin_nontemporal_load((const FSTX_GLOBAL v4u_anywhere *)p);
@@ -331,6 +386,10 @@ template <bool kKeep> struct GatherMem {
     }
     __device__ __forceinline__ void store16(char *p, fstx_gather::Vec16 v) {
         st_stream(v4u{v.w[0], v.w[1], v.w[2], v.w[3]}, reinterpret_cast<v4u *>(p));
+    }
+    // sixteen bytes at any address
+    __device__ __forceinline__ void store16_any(char *p, fstx_gather::Vec16 v) {
+        __builtin_nontemporal_store(v4u{v.w[0], v.w[1], v.w[2], v.w[3]}, (FSTX_GLOBAL v4u_anywhere *)p);
     }
     __device__ __forceinline__ void store8(char *p, unsigned char b) { st_global(b, reinterpret_cast<unsigned char *>(p)); }
 };
@@ -633,7 +692,7 @@ struct GatherBatch {
                                         (uint32_t)live[i].seg_bytes, (uint32_t)col, 0};
             };
             fstx_gather::Job job = fstx_gather::make_job(static_cast<char *>(dst) + row * dst_pitch, dst_pitch, row_bytes,
-                                                         part, source(0, 0), 0, m, m > 1 ? equal : 0);
+                                                         part, source(0, 0), 0, m, m > 1 ? equal : 0, min_seg);
             const uint64_t need = (fstx_gather::tiles_of(job) + kXcds - 1) / kXcds * kXcds; // whole eighths
             if (nj == kGatherJobs || (m > 1 && ns + m > kGatherMore) || tiles + need > lim.launch) {
                 int rc = flush();
@@ -768,14 +827,17 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         for (uint64_t row = 0; row < outer; row += rows_per_job) {
             uint64_t rows = outer - row < rows_per_job ? outer - row : rows_per_job;
             uint64_t units = rows * seg_units;
-            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > lim.launch) {
+            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > lim.launch) { // (an upper bound when packed)
                 int rc = flush();
                 if (rc < 0) return rc;
             }
-            t.job[k] = SliceJob{static_cast<char *>(d.dst) + row * seg,
-                                static_cast<const char *>(d.src) + row * pitch,
-                                pitch | ((uint64_t)ul << 56), (uint32_t)seg_units, (uint32_t)units};
-            blocks_of[k] = (blocks_for(units) + kXcds - 1) / kXcds * kXcds; // whole eighths
+            // units under 16 bytes are packed into whole destination vectors when those are aligned
+            char *job_dst = static_cast<char *>(d.dst) + row * seg;
+            const bool packed = ul < 4 && ((uintptr_t)job_dst & (kVecBytes - 1)) == 0;
+            const uint64_t items = packed ? (units + (16u >> ul) - 1) / (16u >> ul) : units;
+            t.job[k] = SliceJob{job_dst, static_cast<const char *>(d.src) + row * pitch,
+                                pitch | ((uint64_t)(ul | (packed ? kPackedUnits : 0u)) << 56), (uint32_t)seg_units, (uint32_t)units};
+            blocks_of[k] = (blocks_for(items) + kXcds - 1) / kXcds * kXcds; // whole eighths
             blocks += blocks_of[k];
             ++k;
         }
@@ -830,10 +892,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         const fstx_join_src one{d.src, d.seg_bytes, d.src_pitch};
         const uint32_t ul = common_unit_log2((uint64_t)(uintptr_t)d.dst | (uint64_t)(uintptr_t)d.src | d.seg_bytes |
                                              d.src_pitch | d.dst_pitch | 16u);
-        // a narrow block in a wide destination with everything on 16-byte boundaries: the plain
-        // 16-byte-unit kernel below has nothing to realign and measured faster on it
-        const bool plain = ul == 4 && fstx_gather::counts_by_rows(d.dst_pitch, d.seg_bytes);
-        if (mode != 0 && !plain && GatherBatch::takes(d.dst_pitch, d.outer, &one, 1)) {
+        if (mode != 0 && GatherBatch::takes(d.dst_pitch, d.outer, &one, 1)) {
             int rc = gather.add(d.dst, d.dst_pitch, d.outer, &one, 1);
             if (rc < 0) return rc;
             continue;

@@ -131,11 +131,29 @@ def test_narrow_blocks_in_wide_rows(sim):
                 assert bad == 0 and same, (segs, gap, dst_mis, bad)
 
 
+def test_tiles_of_many_short_segments(sim):
+    """Segments under 512 bytes: a tile holds from three to sixty-four of them and every lane finds
+    its own.  One source and joins of up to 24, equal and unequal widths, every destination
+    alignment, dense and pitched (gaps below and above a vector, and wide enough for the row-wise
+    count), enough rows for tiles that lie wholly inside the job."""
+    rng = np.random.default_rng(21)
+    cases = [([16], [16]), ([16], [40]), ([17], [90]), ([254], [1016]), ([96], [384]), ([94], [377]), ([511], [2044]),
+             ([254] * 24, [1016] * 24), ([16] * 24, [64] * 24), ([30, 16, 200], [100, 16, 801]), ([254, 300, 17, 254], [1016, 300, 99, 255]),
+             ([100] * 7, [400] * 7), ([48, 48], [200, 4096]), ([510, 16, 510], [2040, 64, 511])]
+    for segs, pitches in cases:
+        rows = max(6, 9000 // sum(segs) + 3)
+        for gap in (0, 0, 1, 15, 16, 40, 3 * sum(segs)):
+            for dst_mis in (0, 1, 9, 15):
+                mis = [int(x) for x in rng.integers(0, 16, len(segs))]
+                bad, same = run_case(sim, rng, rows + int(rng.integers(0, 5)), segs, pitches, mis, dst_mis, gap)
+                assert bad == 0 and same, (segs, pitches, gap, dst_mis, bad)
+
+
 def test_random_geometries(sim):
     rng = np.random.default_rng(13)
     for trial in range(400):
         n = int(rng.choice([1, 1, 1, 2, 3, 5]))
-        segs = [int(rng.integers(16, 3000)) for _ in range(n)]
+        segs = [int(rng.integers(16, 3000 if trial % 2 else 300)) for _ in range(n)]
         if rng.random() < 0.3:
             segs = [segs[0]] * n
         pitches = [s + int(rng.integers(0, 2000)) for s in segs]

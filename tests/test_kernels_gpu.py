@@ -227,6 +227,29 @@ def test_slice_odd_shapes(dev):
                     assert (got[:lead] == 77).all() and (got[lead + want.numel() :] == 77).all(), "wrote outside the shard"
 
 
+def test_segments_under_16_bytes(dev):
+    """Cuts whose segments are shorter than a vector go to the unit kernel: into an aligned dense
+    destination it packs 16 / unit of them into one store, else it moves one unit per lane.
+    Unit sizes 1, 2, 4 and 8 bytes, row counts that leave a ragged last vector, against torch's
+    slicing, with guard elements around every destination."""
+    for shape, dtype, world in [((100_003, 4), torch.int16, 4), ((65_537, 3), torch.uint8, 3), ((9_999, 6), torch.int16, 2),
+                                ((33_333, 2), torch.int64, 2), ((7, 12), torch.uint8, 4), ((50_001, 2, 3), torch.int32, 2),
+                                ((1, 8), torch.int16, 4), ((12_345, 15), torch.uint8, 1)]:
+        t = torch.randint(0, 120, shape, dtype=dtype, device=dev)
+        item = t.element_size()
+        block = -(-shape[1] // world)
+        inner = int(np.prod(shape[2:], dtype=np.int64)) * item
+        for rank in range(world):
+            lo, hi = min(rank * block, shape[1]), min((rank + 1) * block, shape[1])
+            want = t[:, lo:hi].contiguous()
+            for lead in (0, 1, 8 // item if item < 8 else 1):
+                got = torch.full((want.numel() + 64,), 99, dtype=dtype, device=dev)
+                _native.slice_copy(got.data_ptr() + lead * item, t.data_ptr() + lo * inner, shape[0], (hi - lo) * inner,
+                                   shape[1] * inner, stream())
+                assert torch.equal(got[lead : lead + want.numel()].view(want.shape), want), (shape, dtype, rank, lead)
+                assert (got[:lead] == 99).all() and (got[lead + want.numel() :] == 99).all(), "wrote outside the shard"
+
+
 def test_gather_random_geometry_in_one_batch(dev):
     """Byte-level sweep of the gather kernel: segment lengths from the shortest it takes (16
     bytes; 9 and 15 go to the small-unit kernel) over the tile size and its fractions, odd
