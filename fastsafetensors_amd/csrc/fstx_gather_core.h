@@ -84,8 +84,9 @@ constexpr uint32_t kTile = kLanes * kVec; // destination bytes per wavefront
 constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two segments
 
 // Tile order of every job (a tile = the 1 KiB a wavefront writes; the copy kernels use the same
-// order).  Workgroups reach the eight dies round-robin
-// (workgroup b runs on die b % 8) and every die has its own L2, so in dispatch order the two
+// order).  Workgroups reach the dies of the device round-robin (eight on a whole MI355X: workgroup
+// b runs on die b % 8; four, two or one when the device is a partition of it -- the launch says
+// how many) and every die has its own L2, so in dispatch order the two
 // tiles either side of a shared line would sit on different dies and the line would be fetched
 // from HBM twice, or a destination line written in two parts.  The tiles are therefore dealt out
 // in chunks of 8 x 256: within a chunk die d takes tiles [256 d, 256 d + 256) one after the
@@ -94,20 +95,20 @@ constexpr uint32_t kMinSeg = 16;          // a vector then overlaps at most two 
 // in step (one contiguous eighth of the job per die measured up to 10 % slower on jobs of
 // 100 MB, and 20 % slower when the eighths alias on the channels).  Jobs in which nothing is
 // shared -- everything on cache-line boundaries -- take the same order: it measured 0-2 % faster
-// than dispatch order on them too.  The last, partial chunk is dealt out in eighths.  A job
-// takes ceil(n_tiles / 8) * 8 workgroups; false = an idle one.
-constexpr uint32_t kDies = 8;
+// than dispatch order on them too.  The last, partial chunk is dealt out in equal parts.  A job
+// takes ceil(n_tiles / dies) * dies workgroups; false = an idle one.  One die: dispatch order.
+constexpr uint32_t kMaxDiesLog2 = 3; // eight dies at most; what a launch is told comes from the device (see dies_log2 on the host side)
 constexpr uint32_t kRunLog2 = 8;
-FSTX_HD bool tile_for_die(uint32_t lb, uint32_t n_tiles, uint32_t &tile) {
-    constexpr uint32_t chunk = kDies << kRunLog2;
+FSTX_HD bool tile_for_die(uint32_t lb, uint32_t n_tiles, uint32_t dies_log2, uint32_t &tile) {
+    const uint32_t dies = 1u << dies_log2, chunk = dies << kRunLog2;
     const uint32_t full = n_tiles & ~(chunk - 1);
     if (lb < full) {
-        tile = (lb & ~(chunk - 1)) | ((lb & (kDies - 1)) << kRunLog2) | ((lb / kDies) & ((1u << kRunLog2) - 1));
+        tile = (lb & ~(chunk - 1)) | ((lb & (dies - 1)) << kRunLog2) | ((lb >> dies_log2) & ((1u << kRunLog2) - 1));
         return true;
     }
-    const uint32_t per_die = (n_tiles - full + kDies - 1) / kDies;
-    const uint32_t l = lb - full, turn = l / kDies;
-    tile = full + (l % kDies) * per_die + turn;
+    const uint32_t per_die = (n_tiles - full + dies - 1) >> dies_log2;
+    const uint32_t l = lb - full, turn = l >> dies_log2;
+    tile = full + (l & (dies - 1)) * per_die + turn;
     return turn < per_die && tile < n_tiles;
 }
 

@@ -29,6 +29,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "fstx.h"
 #include "fstx_gather_core.h"
 #include "fstx_internal.h"
@@ -57,7 +60,6 @@ template <typename T> __device__ __forceinline__ void st_global(T v, T *p) { *(F
 #define FSTX_BLOCK 64
 #endif
 constexpr int kBlock = FSTX_BLOCK; // lanes per workgroup
-constexpr uint32_t kXcds = 8;      // accelerator dies; workgroup b is dispatched to die b % 8
 constexpr int kVecBytes = 16;      // bytes moved per lane per step
 
 // ---------------------------------------------------------------- job tables
@@ -120,9 +122,39 @@ __device__ __forceinline__ uint32_t find_job(const Table &t, uint32_t granule_lo
     return (t.owner[g >> 2] >> ((g & 3) * 8)) & 0xffu;
 }
 
-// Host side: lays the jobs' workgroup counts out on granules; returns the grid size.
+// Dies the current device deals workgroups out to, as log2: its compute units / 32 (a die of an
+// MI355X has 32 of them active, so a whole device gives 8 and its partitions 4, 2 or 1), 8 when
+// the runtime does not say; FSTX_DIES overrides it (1, 2, 4 or 8; measurements and tests).  Any
+// value gives the right bytes -- the tile order is a permutation for each -- the right one keeps
+// neighbouring tiles on one die.
+inline uint32_t dies_log2() {
+    static std::atomic<int> cache[64];
+    static std::once_flag once;
+    std::call_once(once, [] {
+        for (auto &c : cache) c.store(-1);
+    });
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fstx_gather::kMaxDiesLog2;
+    int got = cache[dev].load(std::memory_order_relaxed);
+    if (got >= 0) return (uint32_t)got;
+    uint32_t dies = 8;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) dies = (uint32_t)cus / 32;
+    if (const char *e = getenv("FSTX_DIES")) dies = (uint32_t)strtoul(e, nullptr, 10);
+    uint32_t log2 = 0;
+    while (log2 < fstx_gather::kMaxDiesLog2 && (2u << log2) <= dies) ++log2;
+    cache[dev].store((int)log2, std::memory_order_relaxed);
+    return log2;
+}
+inline uint64_t pad_to_dies(uint64_t workgroups) {
+    const uint64_t d = 1ull << dies_log2();
+    return (workgroups + d - 1) / d * d;
+}
+
+// Host side: lays the jobs' workgroup counts out on granules; returns the grid size and the
+// kernels' leading argument (granule_log2 | dies_log2 << 8).
 template <typename Table>
-inline uint64_t plan_grid(Table &t, const uint64_t *blocks_of, uint32_t n, uint32_t *granule_log2) {
+inline uint64_t plan_grid(Table &t, const uint64_t *blocks_of, uint32_t n, uint32_t *launch_word) {
     uint32_t gl = 0;
     for (;; ++gl) {
         uint64_t need = 0;
@@ -137,7 +169,7 @@ inline uint64_t plan_grid(Table &t, const uint64_t *blocks_of, uint32_t n, uint3
         for (uint64_t k = 0; k < span; ++k) owner[granule + k] = (uint8_t)i;
         granule += span;
     }
-    *granule_log2 = gl;
+    *launch_word = gl | dies_log2() << 8;
     return granule << gl;
 }
 
@@ -162,9 +194,10 @@ __device__ __forceinline__ uint32_t from_next_lane(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x130 /* wave_shl:1 */, 0xf, 0xf, false);
 }
 
-__global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_log2,
+__global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t launch_word,
                                                           const JobTable<RealignJob> t) {
     const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
     const uint32_t ji = find_job(t, granule_log2, b);
     const RealignJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
@@ -193,7 +226,7 @@ __global__ __launch_bounds__(kBlock) void realign_kernel(const uint32_t granule_
     // die, in the tile order of tile_for_die (which also measured faster than dispatch order
     // when nothing is shared).
     uint32_t tile;
-    const bool tile_live = tile_for_die(lb, (uint32_t)((nvec + kBlock - 1) / kBlock), tile);
+    const bool tile_live = tile_for_die(lb, (uint32_t)((nvec + kBlock - 1) / kBlock), dies_log2, tile);
     const uint64_t j = (uint64_t)tile * kBlock + threadIdx.x;
     if (m == 0) {
         // source vectors are aligned: a plain streaming copy
@@ -280,9 +313,10 @@ __device__ __forceinline__ void slice_units_packed(const SliceJob &job, uint32_t
 
 constexpr uint32_t kPackedUnits = 0x80; // in the unit byte of SliceJob::pitch_unit: slice_units_packed
 
-__global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_log2,
+__global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t launch_word,
                                                         const JobTable<SliceJob> t) {
     const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
     const uint32_t ji = find_job(t, granule_log2, b);
     const SliceJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
@@ -292,7 +326,7 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t granule_lo
     const uint32_t items = (uint32_t)(((uint64_t)job.total_units + (1u << per_log2) - 1) >> per_log2);
     // neighbouring workgroups on the same die, in the tile order of tile_for_die
     uint32_t tile;
-    if (!tile_for_die(lb, (items + kBlock - 1) / kBlock, tile)) return;
+    if (!tile_for_die(lb, (items + kBlock - 1) / kBlock, dies_log2, tile)) return;
     const uint64_t u64 = (uint64_t)tile * kBlock + threadIdx.x;
     if (u64 >= items) return; // also retires the idle workgroups of a job's last granule
     const uint32_t u = (uint32_t)u64;
@@ -329,14 +363,15 @@ __device__ __forceinline__ void slice2d_units(const Slice2dJob &job, uint32_t u)
     st_stream(ld_stream(src), dst);
 }
 
-__global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t granule_log2,
+__global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t launch_word,
                                                           const JobTable<Slice2dJob> t) {
     const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
     const uint32_t ji = find_job(t, granule_log2, b);
     const Slice2dJob job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
     uint32_t tile;
-    if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, tile)) return;
+    if (!tile_for_die(lb, (job.total_units + kBlock - 1) / kBlock, dies_log2, tile)) return;
     const uint64_t u64 = (uint64_t)tile * kBlock + threadIdx.x;
     if (u64 >= job.total_units) return;
     const uint32_t u = (uint32_t)u64;
@@ -403,8 +438,9 @@ struct GatherTable : JobTable<fstx_gather::Job, kGatherJobs, 1024> {
 static_assert(sizeof(GatherTable) + 32 <= 4096, "kernel arguments are limited to 4 KiB");
 
 template <bool kMulti, bool kPitched, bool kKeep>
-__global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2, const GatherTable t) {
+__global__ __launch_bounds__(64) void gather_kernel(const uint32_t launch_word, const GatherTable t) {
     const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
     const uint32_t ji = find_job(t, granule_log2, b);
     const fstx_gather::Job job = t.fetch(ji);
     const uint32_t lb = b - t.first_block[ji];
@@ -412,7 +448,7 @@ __global__ __launch_bounds__(64) void gather_kernel(const uint32_t granule_log2,
     // the same die (tile_for_die)
     const uint32_t n_tiles = (job.nvec + fstx_gather::kLanes - 1) / fstx_gather::kLanes;
     uint32_t tile;
-    if (!tile_for_die(lb, n_tiles, tile)) return; // idle padding of the job's grid
+    if (!tile_for_die(lb, n_tiles, dies_log2, tile)) return; // idle padding of the job's grid
     GatherMem<kKeep> mem;
     fstx_gather::gather_lane<kMulti, kPitched>(job, t.more, tile, threadIdx.x, mem);
 }
@@ -558,9 +594,10 @@ __device__ __forceinline__ void convert_span(const ConvertJob &job, uint32_t lb)
     }
 }
 
-__global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t granule_log2,
+__global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t launch_word,
                                                           const JobTable<ConvertJob> t) {
     const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
     const uint32_t ji = find_job(t, granule_log2, b);
     const ConvertJob job = t.fetch(ji);
     uint32_t lb = b - t.first_block[ji];
@@ -568,7 +605,7 @@ __global__ __launch_bounds__(kBlock) void convert_kernel(const uint32_t granule_
         const uint32_t per_block_log2 = 7 + (job.src_type < 2 ? job.src_type : 2); // 64 lanes x 16 bytes of f64 / f32 / 16-bit
         const uint32_t n_tiles = (uint32_t)((job.n_elems + (1ull << per_block_log2) - 1) >> per_block_log2);
         uint32_t tile;
-        if (!tile_for_die(lb, n_tiles, tile)) return;
+        if (!tile_for_die(lb, n_tiles, dies_log2, tile)) return;
         lb = tile;
     }
 #define FSTX_CONVERT(S, D) \
@@ -693,7 +730,7 @@ struct GatherBatch {
             };
             fstx_gather::Job job = fstx_gather::make_job(static_cast<char *>(dst) + row * dst_pitch, dst_pitch, row_bytes,
                                                          part, source(0, 0), 0, m, m > 1 ? equal : 0, min_seg);
-            const uint64_t need = (fstx_gather::tiles_of(job) + kXcds - 1) / kXcds * kXcds; // whole eighths
+            const uint64_t need = pad_to_dies(fstx_gather::tiles_of(job));
             if (nj == kGatherJobs || (m > 1 && ns + m > kGatherMore) || tiles + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
@@ -750,7 +787,7 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
         if ((s < o + d.nbytes) && (o < s + d.nbytes)) return -FSTX_E_INVAL; // overlap
         for (uint64_t done = 0; done < d.nbytes; done += piece) {
             const uint64_t len = d.nbytes - done < piece ? d.nbytes - done : piece;
-            const uint64_t need = (blocks_for(len / kVecBytes) + kXcds - 1) / kXcds * kXcds;
+            const uint64_t need = pad_to_dies(blocks_for(len / kVecBytes));
             if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
@@ -827,7 +864,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         for (uint64_t row = 0; row < outer; row += rows_per_job) {
             uint64_t rows = outer - row < rows_per_job ? outer - row : rows_per_job;
             uint64_t units = rows * seg_units;
-            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + kXcds > lim.launch) { // (an upper bound when packed)
+            if (k == FSTX_BATCH_MAX || blocks + blocks_for(units) + 8 > lim.launch) { // (an upper bound when packed)
                 int rc = flush();
                 if (rc < 0) return rc;
             }
@@ -837,7 +874,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
             const uint64_t items = packed ? (units + (16u >> ul) - 1) / (16u >> ul) : units;
             t.job[k] = SliceJob{job_dst, static_cast<const char *>(d.src) + row * pitch,
                                 pitch | ((uint64_t)(ul | (packed ? kPackedUnits : 0u)) << 56), (uint32_t)seg_units, (uint32_t)units};
-            blocks_of[k] = (blocks_for(items) + kXcds - 1) / kXcds * kXcds; // whole eighths
+            blocks_of[k] = pad_to_dies(blocks_for(items));
             blocks += blocks_of[k];
             ++k;
         }
@@ -903,14 +940,14 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         for (uint64_t row = 0; row < d.outer; row += rows_per_job) {
             const uint64_t rows = d.outer - row < rows_per_job ? d.outer - row : rows_per_job;
             const uint64_t units = rows * seg_units;
-            if (k == kJobs || blocks + blocks_for(units) + kXcds > lim.launch) {
+            if (k == kJobs || blocks + blocks_for(units) + 8 > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;
             }
             t.job[k] = Slice2dJob{static_cast<char *>(d.dst) + row * d.dst_pitch,
                                   static_cast<const char *>(d.src) + row * d.src_pitch,
                                   d.src_pitch, d.dst_pitch, (uint32_t)seg_units, (uint32_t)units, ul, 0, 0, 0};
-            blocks_of[k] = (blocks_for(units) + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
+            blocks_of[k] = pad_to_dies(blocks_for(units));
             blocks += blocks_of[k];
             ++k;
         }
@@ -1010,7 +1047,7 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         const uint64_t piece = lim.job * per_block; // elements one job may take
         for (uint64_t done = 0; done < d.n_elems; done += piece) {
             const uint64_t len = d.n_elems - done < piece ? d.n_elems - done : piece;
-            const uint64_t need = ((len + per_block - 1) / per_block + kXcds - 1) / kXcds * kXcds; // dealt out to the dies in eights
+            const uint64_t need = pad_to_dies((len + per_block - 1) / per_block);
             if (k == FSTX_BATCH_MAX || sum + need > lim.launch) {
                 int rc = flush();
                 if (rc < 0) return rc;

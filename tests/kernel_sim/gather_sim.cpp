@@ -90,7 +90,12 @@ struct SimMem {
     }
 };
 
+uint32_t g_dies_log2 = 3;
+
 } // namespace
+
+// dies the simulated launch deals its tiles out to: 1 << log2, log2 in 0..3
+extern "C" void fstx_sim_set_dies_log2(uint32_t log2) { g_dies_log2 = log2 > kMaxDiesLog2 ? kMaxDiesLog2 : log2; }
 
 // Runs one job: `n` sources (src[i], seg[i], pitch[i]) into dst rows `dst_pitch` apart.
 // Returns 0 when every access was legal and every payload byte was written exactly once,
@@ -120,9 +125,10 @@ extern "C" int64_t fstx_gather_sim(char *dst, uint64_t dst_capacity_before, uint
     const bool multi = n > 1 || general, pitched = dst_pitch != col || general;
     // workgroup by workgroup in the order the kernel deals tiles out to the dies; a tile that is
     // skipped or visited twice shows up as payload bytes written never or twice
-    for (uint64_t lb = 0; lb < (tiles + kDies - 1) / kDies * kDies; ++lb) {
+    const uint64_t dies = 1ull << g_dies_log2;
+    for (uint64_t lb = 0; lb < (tiles + dies - 1) / dies * dies; ++lb) {
         uint32_t t;
-        if (!tile_for_die((uint32_t)lb, (uint32_t)tiles, t)) continue;
+        if (!tile_for_die((uint32_t)lb, (uint32_t)tiles, g_dies_log2, t)) continue;
         for (uint32_t lane = 0; lane < kLanes; ++lane) {
             if (multi && pitched) gather_lane<true, true>(jb, more.data(), (uint32_t)t, lane, mem);
             else if (multi) gather_lane<true, false>(jb, more.data(), (uint32_t)t, lane, mem);
@@ -140,10 +146,11 @@ extern "C" int64_t fstx_gather_sim(char *dst, uint64_t dst_capacity_before, uint
 // The tile a workgroup takes (tile_for_die), for all workgroups of a job of n_tiles tiles:
 // out[lb] = tile, or 0xffffffff for an idle workgroup.  Returns the number of workgroups.
 extern "C" uint64_t fstx_tile_order_sim(uint32_t n_tiles, uint32_t *out) {
-    const uint64_t groups = ((uint64_t)n_tiles + kDies - 1) / kDies * kDies;
+    const uint64_t dies = 1ull << g_dies_log2;
+    const uint64_t groups = ((uint64_t)n_tiles + dies - 1) / dies * dies;
     for (uint64_t lb = 0; lb < groups; ++lb) {
         uint32_t t = 0;
-        out[lb] = tile_for_die((uint32_t)lb, n_tiles, t) ? t : 0xffffffffu;
+        out[lb] = tile_for_die((uint32_t)lb, n_tiles, g_dies_log2, t) ? t : 0xffffffffu;
     }
     return groups;
 }

@@ -33,6 +33,7 @@ def sim():
                                     ctypes.POINTER(ctypes.c_uint64), ctypes.c_uint32, ctypes.c_int]
     lib.fstx_div_magic_sim.restype = ctypes.c_uint32
     lib.fstx_div_magic_sim.argtypes = [ctypes.c_uint32, ctypes.c_uint64]
+    lib.fstx_sim_set_dies_log2.argtypes = [ctypes.c_uint32]
     lib.fstx_tile_order_sim.restype = ctypes.c_uint64
     lib.fstx_tile_order_sim.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
     return lib
@@ -164,27 +165,51 @@ def test_random_geometries(sim):
         assert bad == 0 and same, (trial, segs, pitches, rows, gap, mis, bad)
 
 
+@pytest.mark.parametrize("dies", [8, 4, 2, 1])
 @pytest.mark.parametrize("n_tiles", [1, 7, 8, 9, 255, 2047, 2048, 2049, 2056, 4095, 4096, 6000, 3 * 2048 + 1, 100_003])
-def test_tile_order_visits_every_tile_once_and_keeps_neighbours_on_a_die(sim, n_tiles):
-    out = np.empty((n_tiles + 7) // 8 * 8, dtype=np.uint32)
-    groups = sim.fstx_tile_order_sim(n_tiles, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
+def test_tile_order_visits_every_tile_once_and_keeps_neighbours_on_a_die(sim, n_tiles, dies):
+    """For a device of 8, 4, 2 dies, and one die (where the order is the dispatch order)."""
+    sim.fstx_sim_set_dies_log2(dies.bit_length() - 1)
+    try:
+        out = np.empty((n_tiles + dies - 1) // dies * dies, dtype=np.uint32)
+        groups = sim.fstx_tile_order_sim(n_tiles, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
+    finally:
+        sim.fstx_sim_set_dies_log2(3)
     assert groups == out.size
     live = out[out != 0xFFFFFFFF]
     assert live.size == n_tiles and np.array_equal(np.sort(live), np.arange(n_tiles, dtype=np.uint32))
-    # workgroup b runs on die b % 8: a die's tiles come in runs of consecutive tiles (256 long in whole
+    # workgroup b runs on die b % dies: a die's tiles come in runs of consecutive tiles (256 long in whole
     # chunks), in ascending order, so a line shared by two neighbouring tiles is used twice by one die
+    chunk = 256 * dies
     die_of = np.empty(n_tiles, dtype=np.int64)
     idx = np.nonzero(out != 0xFFFFFFFF)[0]
-    die_of[out[idx]] = idx % 8
+    die_of[out[idx]] = idx % dies
     changes = int(np.count_nonzero(np.diff(die_of)))
-    assert changes <= 8 * (n_tiles // 2048 + 1)
-    for d in range(8):
-        mine = out[d::8]
+    assert changes <= dies * (n_tiles // chunk + 1)
+    for d in range(dies):
+        mine = out[d::dies]
         mine = mine[mine != 0xFFFFFFFF].astype(np.int64)
         assert np.all(np.diff(mine) > 0)
-    # all dies work inside one window of 2048 tiles at a time
-    full = n_tiles // 2048 * 2048
-    assert np.array_equal(out[:full] // 2048, np.arange(full) // 2048)
+    # all dies work inside one window of 256 x dies tiles at a time
+    full = n_tiles // chunk * chunk
+    assert np.array_equal(out[:full] // chunk, np.arange(full) // chunk)
+    if dies == 1:
+        assert np.array_equal(out, np.arange(n_tiles, dtype=np.uint32))
+
+
+@pytest.mark.parametrize("dies_log2", [0, 1, 2])
+def test_jobs_on_a_partitioned_device(sim, dies_log2):
+    """The same bytes whatever number of dies the launch is dealt out to."""
+    sim.fstx_sim_set_dies_log2(dies_log2)
+    try:
+        rng = np.random.default_rng(30 + dies_log2)
+        for segs, pitches, rows, gap in [([2046], [8180], 700, 0), ([254] * 5, [1016] * 5, 60, 0), ([94], [377], 300, 4000),
+                                         ([1022, 254, 254], [4090, 1018, 1018], 40, 7)]:
+            mis = [int(x) for x in rng.integers(0, 16, len(segs))]
+            bad, same = run_case(sim, rng, rows, segs, pitches, mis, int(rng.integers(0, 16)), gap)
+            assert bad == 0 and same, (segs, rows, gap, bad)
+    finally:
+        sim.fstx_sim_set_dies_log2(3)
 
 
 def test_division_by_multiplication_is_exact(sim):

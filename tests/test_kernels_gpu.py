@@ -547,3 +547,52 @@ def test_joins_of_random_geometry_small_and_large(dev):
             col += s
         torch.cuda.synchronize()
         assert torch.equal(dst, want), case
+
+
+_PARTITION_CHECK = r"""
+import sys, torch
+from fastsafetensors_amd import _native
+dev = torch.device("cuda:0")
+st = torch.cuda.current_stream().cuda_stream
+g = torch.Generator(device=dev).manual_seed(5)
+# realign copy, shifted source, a few thousand tiles
+src = torch.randint(0, 255, (5_000_011,), dtype=torch.uint8, device=dev, generator=g)
+dst = torch.zeros(5_000_000, dtype=torch.uint8, device=dev)
+_native.realign_copy(dst.data_ptr(), src.data_ptr() + 7, dst.numel(), st)
+assert torch.equal(dst, src[7 : 7 + dst.numel()])
+# aligned column cut (slice kernel), odd column cut (gather kernel), short segments, a narrow block in wide rows, a join
+t = torch.randint(-30000, 30000, (3000, 4096), dtype=torch.int16, device=dev, generator=g)
+for lo, hi in ((1024, 2048), (1001, 2024), (40, 167)):
+    out = torch.empty((3000, hi - lo), dtype=torch.int16, device=dev)
+    _native.slice_copy(out.data_ptr(), t.data_ptr() + 2 * lo, 3000, 2 * (hi - lo), 8192, st)
+    assert torch.equal(out, t[:, lo:hi]), (lo, hi)
+wide = torch.zeros((3000, 1500), dtype=torch.int16, device=dev)
+_native.slice_copy2d_batch([(wide.data_ptr() + 2 * 33, t.data_ptr() + 2 * 5, 3000, 2 * 47, 8192, 3000)], st)
+assert torch.equal(wide[:, 33:80], t[:, 5:52]) and not wide[:, :33].any() and not wide[:, 80:].any()
+parts = [torch.randint(0, 255, (2000, 1016), dtype=torch.uint8, device=dev, generator=g) for _ in range(5)]
+joined = torch.empty((2000, 5 * 254), dtype=torch.uint8, device=dev)
+_native.join_copy(joined.data_ptr(), 2000, [(p.data_ptr() + 254, 254, 1016) for p in parts], st)
+assert torch.equal(joined, torch.cat([p[:, 254:508] for p in parts], dim=1))
+# down-cast
+f = torch.randn(1_000_003, device=dev, generator=g)
+h = torch.empty(f.numel(), dtype=torch.bfloat16, device=dev)
+_native.convert_batch([(h.data_ptr(), f.data_ptr(), f.numel(), _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["BF16"])], st)
+assert torch.equal(h.view(torch.int16), f.to(torch.bfloat16).view(torch.int16))
+torch.cuda.synchronize()
+print("ok")
+"""
+
+
+@pytest.mark.parametrize("dies", ["1", "2", "4"])
+def test_kernels_on_a_device_with_fewer_dies(dies):
+    """The tile order follows the number of dies of the device (compute units / 32; a partition of
+    the chip has 4, 2 or 1).  FSTX_DIES stands in for such a device: the same bytes must come out.
+    The library reads it once per process, hence a process of its own."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, FSTX_DIES=dies, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    proc = subprocess.run([sys.executable, "-c", _PARTITION_CHECK], env=env, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("ok"), proc.stdout + proc.stderr
