@@ -851,6 +851,64 @@ def bench_kernels(steps: int, warmup: int) -> Dict[str, dict]:
         "launches_timed": len(conv_times), "avg_launch_ms": conv_ms, "bytes_per_launch": 6 * per * 48,
         "achieved_GBps": 6 * per * 48 / 1e6 / conv_ms,
     }
+    # -- the remaining variants of the kernels, one row each: the realign copy with its source, then its
+    #    destination, 16 bytes into a cache line; two more conversions; the gather kernel with a pitched
+    #    destination (one source: a column block into a slightly wider tensor; several: a join into one)
+    variants = {}
+
+    def vrow(label, kernel, nb, launch, check=None):
+        launch()
+        ms = timed([launch] * max(3, steps))
+        if check is not None and not check():
+            raise SystemExit(f"bench: {label}: wrong bytes")
+        variants[label] = {"kernel": kernel, "avg_launch_ms": sum(ms) / len(ms), "bytes_per_launch": nb,
+                           "achieved_GBps": nb / 1e6 / (sum(ms) / len(ms))}
+
+    half = 1 << 29
+    vrow("realign copy of 512 MiB, source 16 bytes into a cache line", "realign_kernel", 2 * half,
+         lambda: _native.realign_copy(dst.data_ptr(), window.data_ptr() + 16, half, stream),
+         lambda: torch.equal(dst[:half], window[16 : 16 + half]))
+    vrow("realign copy of 512 MiB, destination 16 bytes into a cache line", "realign_kernel", 2 * half,
+         lambda: _native.realign_copy(dst.data_ptr() + 16, window.data_ptr(), half, stream),
+         lambda: torch.equal(dst[16 : 16 + half], window[:half]))
+    vrow("realign copy of 512 MiB, source shifted by 3 bytes, destination 16 bytes into a cache line", "realign_kernel", 2 * half,
+         lambda: _native.realign_copy(dst.data_ptr() + 16, window.data_ptr() + 3, half, stream),
+         lambda: torch.equal(dst[16 : 16 + half], window[3 : 3 + half]))
+    n16 = cal // 2 // 48 // 64 * 64
+    src16 = window[:cal].view(torch.float16)
+    src16.copy_(torch.randn(src16.numel() // 64, device=dev, dtype=torch.float16).repeat(64))  # finite values
+    dst8 = dst[: cal // 2]
+    cj = [(dst8.data_ptr() + i * n16, src16.data_ptr() + 2 * i * n16, n16, _native.ELEM_TYPES["F16"], _native.ELEM_TYPES["F8_E4M3"])
+          for i in range(48)]
+    vrow(f"fp16 -> fp8 e4m3, 48 tensors of {n16} elements per launch", "convert_kernel", 3 * n16 * 48,
+         lambda: _native.convert_batch(cj, stream),
+         lambda: torch.equal(dst8[: 1 << 22].view(torch.int8), src16[: 1 << 22].to(torch.float8_e4m3fn).view(torch.int8)))
+    src32b = window[:cal].view(torch.float32)
+    src32b.copy_(torch.randn(src32b.numel() // 64, device=dev).repeat(64))
+    cj2 = [(dst16.data_ptr() + 2 * i * per, src32b.data_ptr() + 4 * i * per, per, _native.ELEM_TYPES["F32"], _native.ELEM_TYPES["F16"])
+           for i in range(48)]
+    vrow(f"fp32 -> fp16, 48 tensors of {per} elements per launch", "convert_kernel", 6 * per * 48,
+         lambda: _native.convert_batch(cj2, stream),
+         lambda: torch.equal(dst16[probe], src32b[probe].to(torch.float16).view(torch.int16)))
+    tp = torch.randint(-30000, 30000, (65536, 4090), dtype=torch.int16, device=dev)
+    bw = -(-4090 // world)
+    widep = [torch.zeros((65536, bw + 40), dtype=torch.int16, device=dev) for _ in range(world)]
+    pj = [(widep[r].data_ptr() + 2 * 7, tp.data_ptr() + 2 * r * bw, 65536, 2 * min(bw, 4090 - r * bw), 8180, 2 * (bw + 40)) for r in range(world)]
+    vrow("bf16 [65536, 4090] cut in 4 along dim 1 into columns 7.. of tensors 40 columns wider (pitched destination), 4 ranks per launch",
+         "gather_kernel<one source, pitched>", 2 * 2 * 65536 * 4090, lambda: _native.slice_copy2d_batch(pj, stream),
+         lambda: all(torch.equal(widep[r][:, 7 : 7 + min(bw, 4090 - r * bw)], tp[:, r * bw : (r + 1) * bw]) and not widep[r][:, :7].any()
+                     for r in range(world)))
+    del widep
+    tsj = [torch.randint(0, 100, (32768, 8190), dtype=torch.uint8, device=dev) for _ in range(6)]
+    bj = -(-8190 // world)
+    outp = torch.zeros((32768, 6 * bj + 256), dtype=torch.uint8, device=dev)
+    jp = [(t.data_ptr(), bj, 8190) for t in tsj]
+    vrow("6 x fp8 [32768, 8190], column blocks of rank 0 joined along dim 1 into rows 256 bytes wider (pitched destination)",
+         "gather_kernel<several sources, pitched>", 2 * 32768 * 6 * bj,
+         lambda: _native.join_copy(outp.data_ptr(), 32768, jp, stream, dst_pitch=6 * bj + 256),
+         lambda: torch.equal(outp[:, : 6 * bj], torch.cat([t[:, :bj] for t in tsj], dim=1)) and not outp[:, 6 * bj :].any())
+    del tsj, outp, tp
+    out["variants"] = variants
     avg_ms = sum(times) / len(times)
     out["realign_copy"] = {
         "workload": "C2 GPT-2-medium fp16 data section, 709,646,336 bytes, source shifted by 10 bytes",
@@ -1342,7 +1400,7 @@ def main() -> None:
 
         rows = {name: kern(kernels[name]) for name in ("slice_extract", "row_block_copy", "slice_join_columns", "realign_copy",
                                                         "convert_f32_bf16", "calibration_copy") if name in kernels}
-        for group in ("slice_extract_odd_shapes", "join_odd_columns", "short_segments"):
+        for group in ("slice_extract_odd_shapes", "join_odd_columns", "short_segments", "variants"):
             for label, d in kernels.get(group, {}).items():
                 if "gather_kernel" in d:
                     rows[f"{group}: {label}"] = kern(d["gather_kernel"])

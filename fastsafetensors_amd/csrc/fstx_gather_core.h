@@ -541,7 +541,9 @@ inline Job make_job(char *dst, uint64_t dst_pitch, uint64_t row_bytes, uint64_t 
                     uint32_t nsrc, uint64_t equal_seg, uint64_t min_seg) {
     const uint64_t head = (uint64_t)(uintptr_t)dst & (kVec - 1);
     const uint64_t span = (rows - 1) * dst_pitch + row_bytes;
-    const bool single = nsrc == 1, by_rows = counts_by_rows(dst_pitch, row_bytes), loose = by_rows && single;
+    // one source into a pitched destination is always counted row by row from each row's own first
+    // byte (no vector then holds a gap); several sources only when the gaps are a large part of the rows
+    const bool single = nsrc == 1, loose = single && dst_pitch != row_bytes, by_rows = loose || counts_by_rows(dst_pitch, row_bytes);
     const uint32_t per_row = loose ? loose_vectors_per_row((uint32_t)row_bytes) : vectors_per_row((uint32_t)row_bytes);
     const uint64_t nvec = by_rows ? rows * per_row : (head + span + kVec - 1) / kVec;
     return Job{dst, (uint32_t)dst_pitch, (uint32_t)row_bytes, (uint32_t)rows, (uint16_t)more0, (uint16_t)nsrc,

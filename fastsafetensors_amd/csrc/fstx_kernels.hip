@@ -463,6 +463,9 @@ __global__ __launch_bounds__(64) void gather_kernel(const uint32_t launch_word, 
 // 0x7fc0, fp8 e4m3fn has no infinity (everything from 480 up, and NaN, becomes
 // 0x7f), fp8 e5m2 overflows to infinity; double goes through float first.
 
+#ifndef FSTX_HW_FP8
+#define FSTX_HW_FP8 1
+#endif
 enum : uint32_t { kF64 = 0, kF32 = 1, kF16 = 2, kBF16 = 3, kF8E4M3 = 4, kF8E5M2 = 5 };
 
 struct alignas(32) ConvertJob {
@@ -578,8 +581,32 @@ __device__ __forceinline__ void convert_span(const ConvertJob &job, uint32_t lb)
         src_t in[kPer];
         dst_t out[kPer];
         __builtin_memcpy(in, &raw, 16);
+#if FSTX_HW_FP8
+        if constexpr (D == kF8E4M3 || D == kF8E5M2) {
+            // the hardware's own packed conversion: two values per instruction, nearest-even, overflow
+            // to NaN (e4m3fn) or infinity (e5m2) like torch's.  Only its NaNs are encoded differently
+            // (torch: 0x7f with the sign of the input): those bytes are put right afterwards.
+            uint32_t words[(kPer + 3) / 4] = {};
 #pragma unroll
-        for (uint32_t k = 0; k < kPer; ++k) out[k] = Elem<D>::from_f32(Elem<S>::to_f32(in[k]));
+            for (uint32_t k = 0; k < kPer; k += 2) {
+                const float a = Elem<S>::to_f32(in[k]), b = Elem<S>::to_f32(in[k + 1]);
+                const int old = (int)words[k / 4];
+                if constexpr (D == kF8E4M3) {
+                    words[k / 4] = (uint32_t)((k / 2) & 1 ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, false));
+                } else {
+                    words[k / 4] = (uint32_t)((k / 2) & 1 ? __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, false));
+                }
+                const uint32_t at = 8 * (k & 3);
+                if (a != a) words[k / 4] = (words[k / 4] & ~(0xffu << at)) | ((0x7fu | (f32_bits(a) >> 31) << 7) << at);
+                if (b != b) words[k / 4] = (words[k / 4] & ~(0xff00u << at)) | ((0x7f00u | (f32_bits(b) >> 31) << 15) << at);
+            }
+            __builtin_memcpy(out, words, sizeof out);
+        } else
+#endif
+        {
+#pragma unroll
+            for (uint32_t k = 0; k < kPer; ++k) out[k] = Elem<D>::from_f32(Elem<S>::to_f32(in[k]));
+        }
         if (((uintptr_t)job.dst & (sizeof(out_t) - 1)) == 0) { // uniform: one store at its natural alignment
             out_t packed;
             __builtin_memcpy(&packed, out, sizeof packed);
