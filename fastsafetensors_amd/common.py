@@ -193,9 +193,11 @@ class SafeTensorsMetadata:
         self.tensors: Dict[str, TensorFrame] = {}
         cursor = 0
         items = list(table.items())
-        starts = [entry["data_offsets"][0] for _, entry in items]
-        if any(a > b for a, b in zip(starts, starts[1:])):  # writers emit them in offset order; sort only when not
-            items.sort(key=lambda kv: kv[1]["data_offsets"][0])
+        spans = [tuple(entry["data_offsets"]) for _, entry in items]
+        if any(a > b for a, b in zip(spans, spans[1:])):  # writers emit them in offset order; sort only when not
+            # by (begin, end): an empty tensor shares its offset with its successor and must come first
+            # (the reference sorts by begin alone and then depends on the order of the JSON for such a pair)
+            items.sort(key=lambda kv: tuple(kv[1]["data_offsets"]))
         for name, entry in items:
             frame = TensorFrame.from_buffer(entry)
             begin, end = frame.data_offsets
