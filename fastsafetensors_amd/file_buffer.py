@@ -49,7 +49,12 @@ class FilesBufferOnDevice:
 
     # -- lifetime -----------------------------------------------------------------
     def close(self) -> None:
-        """Free every file buffer; tensors obtained from this object dangle afterwards."""
+        """Free every file buffer; tensors obtained from this object dangle afterwards.
+
+        The memory goes back to the framework's allocator at once.  Work that still reads those
+        tensors must be finished by then, or be queued on the stream that is current on the thread
+        that loads next: the next load orders its copies after that stream only, not after the
+        whole device."""
         for factories in self.rank_loaders.values():
             for factory in factories:
                 factory.free_dev_ptrs()
@@ -148,7 +153,9 @@ class FilesBufferOnDevice:
         """``get_multi_cols`` for many groups in one call -- the q/k/v and gate/up packing of every
         layer, say -- with the copies of all groups batched into a few launches and the results
         in one allocation per file.  (The reference has one call per group,
-        ``file_buffer.py:193-236``; the result of each group is the same.)"""
+        ``file_buffer.py:193-236``; the result of each group is the same.)  The results of one call
+        are views into one allocation per element type and file: the memory of all of them stays
+        allocated until the last of them is dropped."""
         outs: List[Optional[TensorBase]] = [None] * len(groups)
         by_file: Dict[Tuple[int, int], List[int]] = {}
         for i, names in enumerate(groups):
@@ -167,7 +174,9 @@ class FilesBufferOnDevice:
         return outs  # type: ignore[return-value]
 
     def as_dict(self, tensor_shard_dim: "OrderedDict[str, int]") -> Dict[str, TensorBase]:
-        """``{name: dim}`` -> ``{name: tensor}`` with the rule of ``get_sharded``."""
+        """``{name: dim}`` -> ``{name: tensor}`` with the rule of ``get_sharded``.  The blocks cut for
+        consecutive names of one file are views into one allocation per element type: their memory
+        stays allocated until the last of them is dropped (the reference allocates each block on its own)."""
         out: Dict[str, TensorBase] = {}
         run: List[Tuple[str, int]] = []  # consecutive names that live in the same file
         run_of: Optional[Tuple[int, int]] = None

@@ -19,7 +19,7 @@ over it, and knows how to turn a view into what a rank should see:
 from typing import Dict, List, Optional, Tuple
 
 from ._native import DeviceBuffer
-from .common import SafeTensorsMetadata, init_logger, is_debug
+from .common import SafeTensorsMetadata, TensorFrame, init_logger, is_debug
 from .copier.base import CopierInterface, DummyDeviceBuffer
 from .frameworks import FrameworkOpBase, ProcessGroupBase, TensorBase
 from .st_types import Device, DType
@@ -160,24 +160,30 @@ class LazyTensorFactory:
             out[name] = t
         return out
 
+    def _joinable(self, tensor_names: List[str], dim: int) -> List[TensorFrame]:
+        """Frames of tensors that are to be joined along ``dim``: same number of dimensions, same
+        extents everywhere else, and one element type -- the blocks are joined as bytes, and
+        bytes of two types side by side are not a tensor (``torch.cat``, which the reference
+        joins with, would promote them to a common type instead)."""
+        frames = [self.metadata.tensors[name] for name in tensor_names]
+        ref = frames[0]
+        for name, frame in zip(tensor_names, frames):
+            if len(frame.shape) != len(ref.shape):
+                raise Exception(f"rank mismatch: tensor {name} has {frame.shape} vs. {ref.shape} (dim={dim})")
+            for d, extent in enumerate(frame.shape):
+                if d != dim and extent != ref.shape[d]:
+                    raise Exception(f"dim {d} mismatch: tensor {name} has {frame.shape} vs. {list(ref.shape)} (dim={dim})")
+            if frame.dtype != ref.dtype:
+                raise Exception(f"dtype mismatch: tensor {name} is {frame.dtype.value} vs. {ref.dtype.value} of {tensor_names[0]}")
+        return frames
+
     def shuffle_multi_cols(self, pg: ProcessGroupBase, tensor_names: List[str], dim: int) -> TensorBase:
         """The rank's blocks of several tensors joined along ``dim``
         (``tensor_factory.py:194-259``).  The blocks are cut straight into their places in
         the joined tensor by one batched launch (a strided destination when ``dim`` is an
         inner dimension); cutting first and concatenating afterwards remains only for
         tensors that are not in GPU memory."""
-        frames = []
-        ref_shape: Optional[List[int]] = None
-        for name in tensor_names:
-            frame = self.metadata.tensors[name]
-            if ref_shape is None:
-                ref_shape = list(frame.shape)
-            for d, extent in enumerate(frame.shape):
-                if d != dim and extent != ref_shape[d]:
-                    raise Exception(
-                        f"dim {d} mismatch: tensor {name} has {frame.shape} vs. {ref_shape} (dim={dim})"
-                    )
-            frames.append(frame)
+        frames = self._joinable(tensor_names, dim)
         held = [self._held(name, "shuffle_multi_cols") for name in tensor_names]
         rank, world = (0, 1) if pg.size() == 1 else (pg.rank(), pg.size())
         joined = self.framework.extract_shards_joined(list(zip(held, frames)), dim, rank, world)
@@ -193,12 +199,7 @@ class LazyTensorFactory:
         handful of launches for all of them."""
         items = []
         for names in groups:
-            frames = [self.metadata.tensors[n] for n in names]
-            ref = list(frames[0].shape)
-            for n, f in zip(names, frames):
-                for d, extent in enumerate(f.shape):
-                    if d != dim and extent != ref[d]:
-                        raise Exception(f"dim {d} mismatch: tensor {n} has {f.shape} vs. {ref} (dim={dim})")
+            frames = self._joinable(names, dim)
             items.append(list(zip([self._held(n, "shuffle_multi_cols") for n in names], frames)))
         rank, world = (0, 1) if pg.size() == 1 else (pg.rank(), pg.size())
         joined = self.framework.extract_shards_joined_many(items, dim, rank, world)

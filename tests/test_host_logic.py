@@ -100,6 +100,33 @@ def test_world_of_one_returns_views_and_ignores_dim(golden):
     assert FW.get_mem_used() == 0
 
 
+def test_groups_that_cannot_be_joined_as_bytes_are_refused(tmp_path):
+    """get_multi_cols joins the rank's blocks as bytes: tensors of two element types, or of
+    different numbers of dimensions, are refused (the reference's torch.cat would promote the
+    former to a common type; silently joining their bytes would hand back garbage)."""
+    path = str(tmp_path / "mixed.safetensors")
+    save_file({"a.f16": torch.ones(4, 6, dtype=torch.float16), "b.bf16": torch.ones(4, 6, dtype=torch.bfloat16),
+               "c.f16": torch.full((4, 6), 2.0, dtype=torch.float16), "d.f16": torch.ones(4, 6, 1, dtype=torch.float16),
+               "e.i32": torch.ones(4, 6, dtype=torch.int32), "f.f32": torch.ones(4, 6, dtype=torch.float32)}, path)
+    for pg in (SingleGroup(), StubProcessGroup(1, 2)):
+        loader = loader_for(pg)
+        loader.add_filenames({pg.rank(): [path]})
+        bufs = loader.copy_files_to_device()
+        bufs.auto_mem_delete = False
+        with pytest.raises(Exception, match="dtype mismatch: tensor b.bf16 is BF16 vs. F16"):
+            bufs.get_multi_cols(["a.f16", "b.bf16"], dim=0)
+        with pytest.raises(Exception, match="dtype mismatch"):
+            bufs.get_multi_cols_many([["a.f16", "c.f16"], ["e.i32", "f.f32"]], dim=1)
+        with pytest.raises(Exception, match="rank mismatch"):
+            bufs.get_multi_cols(["a.f16", "d.f16"], dim=0)
+        if pg.size() == 1:  # (cutting a rank's blocks needs the GPU)
+            ok = bufs.get_multi_cols(["a.f16", "c.f16"], dim=1).get_raw()
+            assert list(ok.shape) == [4, 12] and ok[:, 6:].eq(2).all()
+        bufs.close()
+        loader.close()
+    assert FW.get_mem_used() == 0
+
+
 def test_push_truth_table(golden):
     path = golden("tiny_gpt2.safetensors")
     ref = load_file(path)
