@@ -48,6 +48,20 @@ bool debug_enabled();
 void debug(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 void note_bounce_bytes(int64_t delta); // process-wide pinned ring accounting
 
+// Named ranges for a profiler's timeline (roctx: they show up in rocprofv3 --marker-trace and in
+// tools that read its output), switched on by FSTX_ROCTX=1: the library then loads
+// librocprofiler-sdk-roctx.so, else libroctx64.so (or what FSTX_ROCTX_LIB names) by itself.  Off, or without that library, a range costs one
+// relaxed load.  Ranges nest per thread and are closed by the destructor.
+struct Range {
+    explicit Range(const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+    ~Range();
+    Range(const Range &) = delete;
+    Range &operator=(const Range &) = delete;
+
+  private:
+    bool open_ = false;
+};
+
 } // namespace fstx_internal
 
 #endif

@@ -697,6 +697,8 @@ struct GatherBatch {
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, tiles_of, nj, &gl);
         if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx gather_kernel: %u jobs, %u sources, %llu tiles%s%s%s", nj, ns, (unsigned long long)tiles,
+                                   multi ? ", joins" : "", pitched ? ", pitched" : "", short_segs ? ", short segments" : "");
         // the leanest variant that serves every job of the launch
         const dim3 g((uint32_t)grid), w(64);
 #define FSTX_GATHER(M, P)                                                                       \
@@ -795,6 +797,7 @@ extern "C" int fstx_realign_copy_batch(const fstx_copy_desc *descs, uint32_t n, 
         uint32_t gl = 0;
         const uint64_t blocks = plan_grid(t, blocks_of, k, &gl);
         if (!grid_fits(blocks)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx realign_kernel: %u jobs, %llu workgroups", k, (unsigned long long)blocks);
         hipLaunchKernelGGL(realign_kernel, dim3((uint32_t)blocks), dim3(kBlock), 0,
                            static_cast<hipStream_t>(stream), gl, t);
         k = 0;
@@ -853,6 +856,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
         if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx slice_kernel: %u jobs, %llu workgroups", k, (unsigned long long)grid);
         hipLaunchKernelGGL(slice_kernel, dim3((uint32_t)grid), dim3(kBlock), 0,
                            static_cast<hipStream_t>(stream), gl, t);
         k = 0;
@@ -932,6 +936,7 @@ extern "C" int fstx_slice_copy2d_batch(const fstx_slice2d_desc *descs, uint32_t 
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
         if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx slice2d_kernel: %u jobs, %llu workgroups", k, (unsigned long long)grid);
         hipLaunchKernelGGL(slice2d_kernel, dim3((uint32_t)grid), dim3(kBlock), 0,
                            static_cast<hipStream_t>(stream), gl, t);
         k = 0;
@@ -1053,6 +1058,7 @@ extern "C" int fstx_convert_batch(const fstx_convert_desc *descs, uint32_t n, vo
         uint32_t gl = 0;
         const uint64_t grid = plan_grid(t, blocks_of, k, &gl);
         if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx convert_kernel: %u jobs, %llu workgroups", k, (unsigned long long)grid);
         hipLaunchKernelGGL(convert_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
                            gl, t);
         k = 0;

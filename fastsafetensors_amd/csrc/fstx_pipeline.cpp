@@ -44,6 +44,7 @@
 #include <thread>
 #include <vector>
 
+#include <dlfcn.h>
 #include <errno.h>
 #include <fcntl.h>
 #include <sched.h>
@@ -680,6 +681,8 @@ struct Worker {
             status.assign(run.size(), -EIO);
             return true;
         }
+        fstx_internal::Range range("fstx O_DIRECT read: %llu MiB at %llu, %zu blocks", (unsigned long long)(want >> 20),
+                                   (unsigned long long)window, run.size());
         uint64_t t0 = now_ns();
         int64_t got = ctx->no_read ? (int64_t)std::min(want, align_up(f.size, kPage) - window)
                                    : pread_full(f.fd_direct, stage, want, window);
@@ -1056,6 +1059,57 @@ void debug(const char *fmt, ...) {
     va_end(ap);
 }
 void note_bounce_bytes(int64_t delta) { g_bounce_bytes.fetch_add(delta); }
+
+namespace {
+typedef int (*roctx_push_t)(const char *);
+typedef int (*roctx_pop_t)(void);
+std::atomic<int> g_roctx_state{0}; // 0 not looked yet, 1 on, -1 off
+roctx_push_t g_roctx_push = nullptr;
+roctx_pop_t g_roctx_pop = nullptr;
+std::once_flag g_roctx_once;
+
+bool roctx_on() {
+    const int st = g_roctx_state.load(std::memory_order_acquire);
+    if (st) return st > 0;
+    std::call_once(g_roctx_once, [] {
+        int found = -1;
+        const char *want = std::getenv("FSTX_ROCTX");
+        if (want && want[0] == '1') {
+            const char *named = std::getenv("FSTX_ROCTX_LIB");
+            // rocprofv3 records the ranges of its own roctx library; the older one serves the older tools
+            const char *names[] = {named && *named ? named : "librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1",
+                                   "libroctx64.so", "libroctx64.so.4"};
+            for (const char *n : names) {
+                void *h = dlopen(n, RTLD_NOW | RTLD_GLOBAL);
+                if (!h) continue;
+                g_roctx_push = reinterpret_cast<roctx_push_t>(dlsym(h, "roctxRangePushA"));
+                g_roctx_pop = reinterpret_cast<roctx_pop_t>(dlsym(h, "roctxRangePop"));
+                if (g_roctx_push && g_roctx_pop) {
+                    found = 1;
+                    break;
+                }
+            }
+            if (found < 0) debug("FSTX_ROCTX=1 but no roctx library could be loaded: no ranges");
+        }
+        g_roctx_state.store(found, std::memory_order_release);
+    });
+    return g_roctx_state.load(std::memory_order_acquire) > 0;
+}
+} // namespace
+
+Range::Range(const char *fmt, ...) {
+    if (!roctx_on()) return;
+    char text[160];
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(text, sizeof text, fmt, ap);
+    va_end(ap);
+    g_roctx_push(text);
+    open_ = true;
+}
+Range::~Range() {
+    if (open_) g_roctx_pop();
+}
 } // namespace fstx_internal
 
 extern "C" {
@@ -1233,6 +1287,8 @@ namespace {
 // every block with that status), so that tearing down is the same in both cases.
 int build_context(fstx_ctx *ctx) {
     const fstx_config &cfg = ctx->cfg;
+    fstx_internal::Range range("fstx build reader: %u threads, %u streams, ring %llu MiB", cfg.n_threads, cfg.n_streams,
+                               (unsigned long long)(ctx->ring_bytes >> 20));
     void *p = nullptr;
     int ring_rc = 0, bound = 0, ring_node = -1;
     uint64_t t_ring = 0;
@@ -1559,6 +1615,8 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
                          void *dev_base, uint64_t dev_capacity, uint64_t dst_off) {
     if (!ctx || (!dev_base && length)) return -FSTX_E_INVAL;
     if (dst_off > dev_capacity || length > dev_capacity - dst_off) return -FSTX_E_RANGE;
+    fstx_internal::Range range("fstx submit_read file %lld: %llu bytes at %llu", (long long)file, (unsigned long long)length,
+                               (unsigned long long)file_off);
     auto req = std::make_shared<Request>();
     {
         std::lock_guard<std::mutex> lk(ctx->table_mutex);
@@ -1616,6 +1674,7 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
 
 int64_t fstx_wait_read(fstx_ctx *ctx, int64_t request) {
     if (!ctx) return -FSTX_E_INVAL;
+    fstx_internal::Range range("fstx wait_read request %lld", (long long)request);
     std::shared_ptr<Request> req;
     {
         std::lock_guard<std::mutex> lk(ctx->table_mutex);

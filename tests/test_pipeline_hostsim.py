@@ -240,6 +240,70 @@ def test_a_failed_build_is_reported_by_whoever_waits(sim, blob):
         sim.fstx_sim_fail_host_allocs(0)
 
 
+_FAKE_ROCTX = r"""
+#include <stdio.h>
+#include <string.h>
+static __thread int depth;
+static int pushes, pops, worst;
+static char first[8][160];
+int roctxRangePushA(const char *m) { int n = __sync_fetch_and_add(&pushes, 1); if (n < 8) strncpy(first[n], m, 159); if (++depth > worst) worst = depth; return depth; }
+int roctxRangePop(void) { __sync_fetch_and_add(&pops, 1); return --depth; }
+void fake_roctx_report(int *a, int *b, int *c, char *names) { *a = pushes; *b = pops; *c = worst; names[0] = 0; for (int i = 0; i < 8 && i < pushes; ++i) { strcat(names, first[i]); strcat(names, "|"); } }
+"""
+
+_ROCTX_CHECK = r"""
+import ctypes, os, sys
+import numpy as np
+sim = ctypes.CDLL(sys.argv[1]); fake = ctypes.CDLL(sys.argv[2], mode=ctypes.RTLD_GLOBAL); path = sys.argv[3]
+from fastsafetensors_amd import _native
+cfg = _native.FstxConfig(ctypes.sizeof(_native.FstxConfig), 0, -1, 3, 2, 64 * 1024, 2, 0, 0, int(sys.argv[4]), 0)
+ctx = ctypes.c_void_p()
+assert sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(ctx)) == 0
+sim.fstx_file_open.restype = ctypes.c_int64; sim.fstx_submit_read.restype = ctypes.c_int64; sim.fstx_wait_read.restype = ctypes.c_int64
+sim.fstx_file_open.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int]
+sim.fstx_submit_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64]
+sim.fstx_wait_read.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+f = sim.fstx_file_open(ctx, path.encode(), 2)
+size = os.path.getsize(path)
+dev = np.zeros(size, dtype=np.uint8)
+req = sim.fstx_submit_read(ctx, f, 0, size, dev.ctypes.data, size, 0)
+assert sim.fstx_wait_read(ctx, req) == size
+assert np.array_equal(dev, np.fromfile(path, dtype=np.uint8))
+sim.fstx_ctx_destroy.argtypes = [ctypes.c_void_p]; sim.fstx_ctx_destroy(ctx)
+a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(); names = ctypes.create_string_buffer(2000)
+fake.fake_roctx_report(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c), names)
+print(a.value, b.value, c.value, names.value.decode())
+"""
+
+
+def test_profiler_ranges_are_named_and_balanced(sim, blob, tmp_path):
+    """FSTX_ROCTX=1: the library loads a roctx library by itself and brackets the build of the reader,
+    every submit, every wait and every O_DIRECT read with a named range; pushes and pops balance on
+    every thread.  Without the switch nothing is loaded and nothing is called.  (A counting stand-in
+    for libroctx64.so, in a process of its own: the switch is read once.)"""
+    import sys
+
+    path, _data = blob
+    src = tmp_path / "fake_roctx.c"
+    src.write_text(_FAKE_ROCTX)
+    lib = str(tmp_path / "libfake_roctx.so")
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O1", "-o", lib, str(src)], check=True)
+    root = os.path.dirname(HERE)
+    for flags in (0, _native.CREATE_ASYNC):
+        for switch, expect_calls in (("1", True), ("0", False)):
+            env = dict(os.environ, FSTX_ROCTX=switch, FSTX_ROCTX_LIB=lib, PYTHONPATH=root)
+            out = subprocess.run([sys.executable, "-c", _ROCTX_CHECK, os.path.join(SIM_DIR, "libfstx_hostsim.so"), lib, path, str(flags)],
+                                 env=env, capture_output=True, text=True, timeout=120)
+            assert out.returncode == 0, out.stderr
+            pushes, pops, worst, names = (out.stdout.strip() + " ").split(" ", 3)
+            if not expect_calls:
+                assert (pushes, pops) == ("0", "0")
+                continue
+            assert int(pushes) == int(pops) >= 4 and int(worst) >= 1
+            assert "fstx build reader: 3 threads, 2 streams" in names and "fstx submit_read file 1" in names
+            assert "fstx wait_read request 1" in names or int(pushes) > 8
+
+
 def test_injected_read_fault(sim, blob):
     path, data = blob
     os.environ["FSTX_FAULT_READ_AFTER"] = "5"
