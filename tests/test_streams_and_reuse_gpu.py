@@ -134,11 +134,11 @@ def test_shared_reader_lives_as_long_as_someone_holds_it(golden):
     path = golden("a.safetensors")
     ring = 4 * 2 * (4096 * 1024 + 4096)
     a = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)
-    a.copier_constructor.reader.wait()  # a loader's reader is built on a helper thread; wait() joins it
+    a.copier_constructor.reader.metrics()  # a loader's reader is built behind its back; asking for the metrics waits for it
     assert _native.bounce_buffer_bytes() == ring
     b = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)          # same settings: same reader
     c = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4, shared_reader=False)
-    b.copier_constructor.reader.wait(), c.copier_constructor.reader.wait()
+    b.copier_constructor.reader.metrics(), c.copier_constructor.reader.metrics()
     assert _native.bounce_buffer_bytes() == 2 * ring
     for ld in (a, b, c):
         ld.add_filenames({0: [path]})
