@@ -335,7 +335,7 @@ def run_load(files: List[str], read_mode: str, threads: int, block_kb: int, veri
     return out
 
 
-def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None) -> dict:
+def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, with_cpu: bool = False) -> dict:
     """Configs C1 (GPT-2-small fp32, 0.5 GB) and C2 (GPT-2-medium fp16, 0.7 GB, header length
     = 2 mod 8) -- the sizes of the reference's published single-file figures
     (docs/amd-perf.md:72-86) -- cold and warm, loader construction to last tensor.  For a file
@@ -413,6 +413,14 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None) ->
             ceiling = co_held if k == "warm_held_reader" else co
             out[k]["copy_only_leg_GBps"] = ceiling["GBps"]
             out[k]["frac_of_copy_only_leg"] = out[k]["GBps"] / ceiling["GBps"]
+    if with_cpu:
+        # the reference's device="cpu" path on the same file, cold and warm
+        drop_cache(files)
+        cc = cpu_baseline(files, cold=True)
+        warm_cache(files)
+        cw = cpu_baseline(files)
+        out["cpu_reference"] = {"kind": cw["kind"], "cold_GBps": cc["value"], "warm_GBps": cw["value"], "cores": cw["cores"],
+                                "defaults_cold_GBps": cc["settings"]["defaults"]["GBps"], "defaults_warm_GBps": cw["settings"]["defaults"]["GBps"]}
     torch.cuda.empty_cache()
     shutil.rmtree(data_dir, ignore_errors=True)
     return out
@@ -1028,7 +1036,7 @@ def cpu_baseline(files: List[str], budget_s: float = 25.0, cold: bool = False) -
 
 
 def bench_whole_load(files: List[str], data_bytes: int, verify, threads: int, block_kb: int, reps: int = 3,
-                     iterate: bool = False) -> dict:
+                     iterate: bool = False, with_cpu: bool = False) -> dict:
     """Warm whole loads (loader construction to last tensor) of a checkpoint whose files sit in
     the page cache or on tmpfs, next to the copy-only leg of the same requests; the first load is
     verified against the generator's checksums.  ``iterate`` adds ``ParallelLoader.iterate_weights``."""
@@ -1047,6 +1055,11 @@ def bench_whole_load(files: List[str], data_bytes: int, verify, threads: int, bl
     if iterate:
         out["iterate_weights"] = bench_iterate_weights(files, threads, verify)
         torch.cuda.empty_cache()
+    if with_cpu:
+        # the reference's device="cpu" path over as many of the files as 12 s allow (page-cache / tmpfs reads)
+        cw = cpu_baseline(files, budget_s=12.0)
+        out["cpu_reference"] = {"kind": cw["kind"], "warm_GBps": cw["value"], "cores": cw["cores"], "sample": cw["sample"],
+                                "defaults_warm_GBps": cw["settings"]["defaults"]["GBps"]}
     return out
 
 
@@ -1227,7 +1240,7 @@ def main() -> None:
 
         small = {}
         for k in ("C1", "C2"):
-            small[k] = bench_small_checkpoint(k, os.path.join(args.dir, k + "_small"), args.threads, write)
+            small[k] = bench_small_checkpoint(k, os.path.join(args.dir, k + "_small"), args.threads, write, with_cpu=not args.skip_cpu_baseline)
             w = small[k]["warm"]
             log(f"[bench] {k}: cold {small[k]['cold']['GBps']:.2f} GB/s (io {small[k]['cold']['io_over_read_only_leg']:.3f} x read-only leg), "
                 f"warm {w['GBps']:.1f} GB/s = {w['frac_of_copy_only_leg']:.3f} of the copy-only leg, held "
@@ -1247,7 +1260,7 @@ def main() -> None:
             tp_files = [r["path"] for r in tp_recs]
             warm_cache(tp_files)
         torch.cuda.empty_cache()
-        c4 = bench_whole_load(tp_files, c4_bytes, c4_sums, args.threads, args.block_kb)
+        c4 = bench_whole_load(tp_files, c4_bytes, c4_sums, args.threads, args.block_kb, with_cpu=not args.skip_cpu_baseline)
         log(f"[bench] C4 whole load (warm): {c4['GBps']:.1f} GB/s in {c4['seconds_to_load']:.3f}s = {c4['frac_of_copy_only_leg']:.3f} of the copy-only leg")
         tp = bench_tp_extract(tp_files, 4, args.threads, args.block_kb)
         log(f"[bench] TP=4 as_dict over the resident checkpoint: {tp['GBps']:.0f} GB/s, seconds per rank {[round(x, 4) for x in tp['seconds_per_rank']]}")
@@ -1268,7 +1281,8 @@ def main() -> None:
             c5_sums: Dict[str, Tuple[int, int]] = {}
             c5_recs, c5_bytes = write("C5", c5_dir, "cuda", False, c5_sums)
             torch.cuda.empty_cache()
-            c5 = bench_whole_load([r["path"] for r in c5_recs], c5_bytes, c5_sums, args.threads, args.block_kb, reps=2, iterate=True)
+            c5 = bench_whole_load([r["path"] for r in c5_recs], c5_bytes, c5_sums, args.threads, args.block_kb, reps=2, iterate=True,
+                                  with_cpu=not args.skip_cpu_baseline)
             shutil.rmtree(c5_dir, ignore_errors=True)
             log(f"[bench] C5 whole load (tmpfs): {c5['GBps']:.1f} GB/s in {c5['seconds_to_load']:.3f}s = {c5['frac_of_copy_only_leg']:.3f} of the copy-only leg; "
                 f"iterate_weights {c5['iterate_weights']['GBps']:.1f} GB/s")
@@ -1420,6 +1434,8 @@ def main() -> None:
                "warm_frac_of_copy_only_leg": r3(sc["warm"]["frac_of_copy_only_leg"]),
                "warm_held_reader_GBps": r3(sc["warm_held_reader"]["GBps"]),
                "warm_held_reader_frac": r3(sc["warm_held_reader"]["frac_of_copy_only_leg"])}
+        if "cpu_reference" in sc:
+            row["cpu_reference_GBps"] = {k2: r3(v) for k2, v in sc["cpu_reference"].items() if k2.endswith("GBps")}
         if "warm_window_layout_realign" in sc:
             row["warm_window_layout_realign_GBps"] = r3(sc["warm_window_layout_realign"]["GBps"])
             row["warm_window_layout_realign_frac"] = r3(sc["warm_window_layout_realign"]["frac_of_copy_only_leg"])
@@ -1429,11 +1445,16 @@ def main() -> None:
                              "tp4_as_dict_GBps": round(tp["GBps"]), "tp4_as_dict_ms_per_rank": [round(1e3 * x, 2) for x in tp["seconds_per_rank"]],
                              "tp4_multi_cols_GBps": round(mc["GBps"]), "tp4_multi_cols_ms_per_rank": [round(1e3 * x, 2) for x in mc["seconds_per_rank"]],
                              "shards_reassembled": tp["tensors_reassembled_and_compared"]}
+    if "cpu_reference" in c4:
+        line["configs"]["C4"]["cpu_reference_GBps"] = {k2: r3(v) for k2, v in c4["cpu_reference"].items() if k2.endswith("GBps")}
     if c5 and "skipped" not in c5:
         line["configs"]["C5"] = {"warm_GBps": r3(c5["GBps"]), "warm_s": r3(c5["seconds_to_load"]), "data_bytes": c5["data_bytes"],
                                  "warm_frac_of_copy_only_leg": r3(c5["frac_of_copy_only_leg"]), "storage": "tmpfs",
                                  "verified_tensors": c5["verified_tensors"],
                                  "iterate_weights_GBps": r3(c5["iterate_weights"]["GBps"])}
+        if "cpu_reference" in c5:
+            line["configs"]["C5"]["cpu_reference_GBps"] = {k2: r3(v) for k2, v in c5["cpu_reference"].items() if k2.endswith("GBps")}
+            line["configs"]["C5"]["cpu_reference_sample"] = c5["cpu_reference"]["sample"]
     else:
         line["configs"]["C5"] = c5
     line["downcast_on_load_GBps"] = {k: r3(v["GBps"]) for k, v in downcast.items() if isinstance(v, dict)}
