@@ -389,7 +389,7 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, wi
         variants["warm_window_layout_realign"] = {"layout": "window"}
     loads = {k: [] for k in variants}
     legs = []
-    for _ in range(4):
+    for _ in range(6):
         legs.append(leg("copy_only", False, reps=2))
         for k, kw in variants.items():
             loads[k] += [run_load(files, "auto", threads, 4096, None, **kw) for _ in range(2)]
@@ -400,7 +400,7 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, wi
     try:
         run_load(files, "auto", threads, 4096, None)  # maps the ring's pages
         held_loads, held_legs = [], []
-        for _ in range(3):
+        for _ in range(5):
             held_legs.append(leg("copy_only", False, reps=2, held=True))
             held_loads += [run_load(files, "auto", threads, 4096, None) for _ in range(2)]
         co_held = max(held_legs, key=lambda r: r["GBps"])

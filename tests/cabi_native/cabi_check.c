@@ -113,7 +113,12 @@ int main(int argc, char **argv) {
     /* ---- a shared context: two users, one ring; ordered after the null stream's work ---- */
     {
         fstx_ctx *a = NULL, *b = NULL;
-        CHECK(fstx_ctx_acquire(&cfg, &a) == 0 && fstx_ctx_acquire(&cfg, &b) == 0 && a == b);
+        /* the first user has it built behind its back; how a context came to be is not part of what it is */
+        fstx_config behind = cfg;
+        behind.flags = FSTX_CREATE_ASYNC;
+        CHECK(fstx_ctx_acquire(&behind, &a) == 0 && fstx_ctx_acquire(&cfg, &b) == 0 && a == b);
+        met.struct_size = sizeof met;
+        CHECK(fstx_get_metrics(a, &met) == 0 && met.create_ns > 0); /* waits for the build */
         const uint64_t ring = fstx_bounce_buffer_bytes();
         CHECK(ring > 0);
         CHECK(hipMemset(arena, 0x11, size + 256) == hipSuccess); /* queued on the null stream ... */
