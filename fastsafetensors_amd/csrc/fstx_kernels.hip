@@ -39,6 +39,7 @@
 namespace {
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef v4u v4u_anywhere __attribute__((aligned(1))); // sixteen bytes at any address
 
 // Every pointer a job carries is device memory.  Saying so (address space 1) lets the
 // compiler emit global_load/global_store instead of flat accesses, which would have to
@@ -343,6 +344,82 @@ __global__ __launch_bounds__(kBlock) void slice_kernel(const uint32_t launch_wor
     }
 }
 
+// Segments under 16 bytes whose rows lie close together (a [N, 4] tensor cut in four: two bytes of
+// every eight): the rows that feed one tile of the destination span a few KiB of source, which the
+// wavefront copies into LDS with whole 16-byte loads -- every line of the source is requested once --
+// and then picks apart: a lane reads the 16 / unit units of its destination vector out of LDS and
+// writes them with one 16-byte store.  One unit per global load, as the other unit paths do it,
+// asks the memory pipeline for each line many times over.
+constexpr uint32_t kStageBytes = 8192;
+
+template <typename Unit>
+__device__ __forceinline__ void units_from_stage(const SliceJob &job, const unsigned char *stage, uint32_t pitch, uint32_t r0,
+                                                 uint32_t q, uint32_t total) {
+    constexpr uint32_t kPer = kVecBytes / sizeof(Unit);
+    const uint32_t seg = job.seg_units * (uint32_t)sizeof(Unit);
+    uint32_t row = q / seg;
+    uint32_t cu = (q - row * seg) / (uint32_t)sizeof(Unit);
+    const uint32_t left = (total - q) / (uint32_t)sizeof(Unit);
+    const uint32_t live = left < kPer ? left : kPer;
+    Unit part[kPer];
+#pragma unroll
+    for (uint32_t k = 0; k < kPer; ++k) {
+        part[k] = Unit{};
+        if (k < live) part[k] = *reinterpret_cast<const Unit *>(stage + (row - r0) * pitch + cu * (uint32_t)sizeof(Unit));
+        if (++cu == job.seg_units) {
+            cu = 0;
+            ++row;
+        }
+    }
+    char *dst = job.dst + q;
+    if (live == kPer) {
+        v4u whole;
+        __builtin_memcpy(&whole, part, sizeof whole);
+        st_stream(whole, reinterpret_cast<v4u *>(dst));
+    } else {
+#pragma unroll
+        for (uint32_t k = 0; k < kPer; ++k)
+            if (k < live) st_global(part[k], reinterpret_cast<Unit *>(dst) + k);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void stage_kernel(const uint32_t launch_word, const JobTable<SliceJob> t) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char stage[]; // as many bytes as the launch's widest window (<= kStageBytes)
+    const uint32_t b = blockIdx.x;
+    const uint32_t granule_log2 = launch_word & 0xffu, dies_log2 = launch_word >> 8;
+    const uint32_t ji = find_job(t, granule_log2, b);
+    const SliceJob job = t.fetch(ji);
+    const uint32_t lb = b - t.first_block[ji];
+    const uint32_t ul = (uint32_t)(job.pitch_unit >> 56) & 7u;
+    const uint32_t pitch = (uint32_t)job.pitch_unit; // a few KiB at most (the host checks)
+    const uint32_t seg = job.seg_units << ul;
+    const uint32_t total = job.total_units << ul;    // destination bytes, below 2^32 (the host cuts jobs accordingly)
+    constexpr uint32_t kTileBytes = kBlock * kVecBytes;
+    uint32_t tile;
+    if (!tile_for_die(lb, (total + kTileBytes - 1) / kTileBytes, dies_log2, tile)) return;
+    const uint32_t d0 = tile * kTileBytes;
+    const uint32_t d1 = total - d0 < kTileBytes ? total : d0 + kTileBytes;
+    const uint32_t r0 = d0 / seg, r1 = (d1 - 1) / seg; // rows that feed this tile
+    const char *win = job.src + (uint64_t)r0 * pitch;
+    const uint32_t window = (r1 - r0) * pitch + seg;   // <= kStageBytes; ends with the last row's segment, inside the block
+    for (uint32_t at = kVecBytes * threadIdx.x; at < window; at += kTileBytes) {
+        if (at + kVecBytes <= window) {
+            *reinterpret_cast<v4u *>(stage + at) = *(const FSTX_GLOBAL v4u_anywhere *)(win + at);
+        } else { // the window's ragged end: byte by byte, never past the last segment
+            for (uint32_t i = at; i < window; ++i) stage[i] = (unsigned char)ld_global(win + i);
+        }
+    }
+    __syncthreads();
+    const uint32_t q = d0 + kVecBytes * threadIdx.x;
+    if (q >= total) return;
+    switch (ul) { // uniform across the workgroup
+    case 3: units_from_stage<uint64_t>(job, stage, pitch, r0, q, total); break;
+    case 2: units_from_stage<uint32_t>(job, stage, pitch, r0, q, total); break;
+    case 1: units_from_stage<uint16_t>(job, stage, pitch, r0, q, total); break;
+    default: units_from_stage<uint8_t>(job, stage, pitch, r0, q, total); break;
+    }
+}
+
 // The same gather with a strided destination: segment `row` is written to
 // dst + row * dst_pitch.  Used to cut the blocks of several tensors straight into one
 // joined tensor along an inner dimension.
@@ -391,7 +468,6 @@ __global__ __launch_bounds__(kBlock) void slice2d_kernel(const uint32_t launch_w
 // tests).  One 16-byte load at the data's own byte address, one aligned 16-byte store; a
 // launch carries up to FSTX_BATCH_MAX jobs and FSTX_BATCH_MAX sources in its arguments.
 
-typedef v4u v4u_anywhere __attribute__((aligned(1)));
 
 // kKeep: the launch holds a job with segments shorter than kShortSeg.  A cache line then holds
 // parts of several segments, which neighbouring lanes and tiles fetch one after the other, and
@@ -863,6 +939,23 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
         blocks = 0;
         return fstx_internal::check_launch("slice_kernel");
     };
+    // the same for cuts that go through LDS (stage_kernel)
+    JobTable<SliceJob> ts;
+    uint64_t blocks_of_s[FSTX_BATCH_MAX];
+    uint64_t blocks_s = 0, stage_bytes = 0;
+    uint32_t ks = 0;
+    auto flush_staged = [&]() -> int {
+        if (ks == 0) return 0;
+        uint32_t gl = 0;
+        const uint64_t grid = plan_grid(ts, blocks_of_s, ks, &gl);
+        if (!grid_fits(grid)) return -FSTX_E_RANGE;
+        fstx_internal::Range range("fstx stage_kernel: %u jobs, %llu workgroups", ks, (unsigned long long)grid);
+        // the less LDS a wavefront holds, the more of them a compute unit runs at once
+        hipLaunchKernelGGL(stage_kernel, dim3((uint32_t)grid), dim3(kBlock), (uint32_t)stage_bytes, static_cast<hipStream_t>(stream), gl, ts);
+        ks = 0;
+        blocks_s = stage_bytes = 0;
+        return fstx_internal::check_launch("stage_kernel");
+    };
     fstx_copy_desc spans[FSTX_BATCH_MAX];
     uint32_t n_spans = 0;
     const Limits lim = limits();
@@ -889,6 +982,28 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
             continue;
         }
         const uint64_t seg_units = seg >> ul;
+        // Short segments in rows that lie close together, into an aligned destination: through LDS, when
+        // the rows that feed one tile of the destination fit the staging buffer.
+        constexpr uint64_t kTileBytes = (uint64_t)kBlock * kVecBytes;
+        const uint64_t window_max = ((kTileBytes / seg + 2) * pitch + seg + kVecBytes - 1) / kVecBytes * kVecBytes;
+        if (ul < 4 && seg < 64 && ((uintptr_t)d.dst & (kVecBytes - 1)) == 0 && window_max <= kStageBytes) {
+            const uint64_t per_job = ((1ull << 32) - 2 * kTileBytes) / seg / 16 * 16; // destination bytes below 2^32; whole vectors per job
+            for (uint64_t row = 0; row < outer; row += per_job) {
+                const uint64_t rows = outer - row < per_job ? outer - row : per_job;
+                const uint64_t need = pad_to_dies(blocks_for(rows * seg / kVecBytes + 1));
+                if (ks == FSTX_BATCH_MAX || blocks_s + need > lim.launch) {
+                    int rc = flush_staged();
+                    if (rc < 0) return rc;
+                }
+                ts.job[ks] = SliceJob{static_cast<char *>(d.dst) + row * seg, static_cast<const char *>(d.src) + row * pitch,
+                                      pitch | ((uint64_t)ul << 56), (uint32_t)seg_units, (uint32_t)(rows * seg_units)};
+                blocks_of_s[ks] = need;
+                blocks_s += need;
+                if (window_max > stage_bytes) stage_bytes = window_max;
+                ++ks;
+            }
+            continue;
+        }
         // rows per job so that the unit index fits 32 bits
         uint64_t rows_per_job = lim.units() / seg_units;
         if (rows_per_job == 0) return -FSTX_E_RANGE; // a single segment of 3 Gi units or more
@@ -912,6 +1027,7 @@ extern "C" int fstx_slice_copy_batch(const fstx_slice_desc *descs, uint32_t n, v
     }
     int rc = flush();
     if (rc < 0) return rc;
+    if ((rc = flush_staged()) < 0) return rc;
     if ((rc = gather.flush()) < 0) return rc;
     return n_spans ? fstx_realign_copy_batch(spans, n_spans, stream) : 0;
 }

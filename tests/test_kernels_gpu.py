@@ -234,7 +234,13 @@ def test_segments_under_16_bytes(dev):
     slicing, with guard elements around every destination."""
     for shape, dtype, world in [((100_003, 4), torch.int16, 4), ((65_537, 3), torch.uint8, 3), ((9_999, 6), torch.int16, 2),
                                 ((33_333, 2), torch.int64, 2), ((7, 12), torch.uint8, 4), ((50_001, 2, 3), torch.int32, 2),
-                                ((1, 8), torch.int16, 4), ((12_345, 15), torch.uint8, 1)]:
+                                ((1, 8), torch.int16, 4), ((12_345, 15), torch.uint8, 1),
+                                # rows close together: staged through LDS (up to the row pitch where the rows of one
+                                # tile no longer fit), rows far apart: one unit per load; segment lengths that do and
+                                # do not divide a tile; the last tile ragged
+                                ((70_001, 8), torch.int16, 8), ((20_011, 24), torch.uint8, 2), ((3_001, 60), torch.uint8, 4),
+                                ((5_003, 1000), torch.uint8, 100), ((4_099, 14), torch.int16, 2), ((1_000_003, 4), torch.uint8, 2),
+                                ((2, 4), torch.int16, 4), ((600, 5), torch.int32, 5), ((513, 16), torch.int16, 4)]:
         t = torch.randint(0, 120, shape, dtype=dtype, device=dev)
         item = t.element_size()
         block = -(-shape[1] // world)
