@@ -1292,8 +1292,8 @@ int build_context(fstx_ctx *ctx) {
     void *p = nullptr;
     int ring_rc = 0, bound = 0, ring_node = -1;
     uint64_t t_ring = 0;
-    std::thread placer([&] {
-        bound = bind_thread_to_node(cfg.numa_node);
+    auto place_ring = [&](bool own_thread) {
+        if (own_thread) bound = bind_thread_to_node(cfg.numa_node); // never the caller's own affinity and policy
         ring_rc = fstx_dev::set_device(cfg.device_id);
         if (ring_rc == 0) ring_rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
         if (ring_rc == 0 && p && cfg.numa_node >= 0) {
@@ -1314,7 +1314,13 @@ int build_context(fstx_ctx *ctx) {
             ctx->ring_ready = true;
         }
         ctx->ready_cv.notify_all();
-    });
+    };
+    std::thread placer;
+    try {
+        placer = std::thread(place_ring, true);
+    } catch (const std::system_error &) {
+        place_ring(false); // no thread to be had: here, unbound
+    }
     int spawn_rc = 0;
     try {
         for (uint32_t t = 0; t < cfg.n_threads; ++t) {
@@ -1334,7 +1340,7 @@ int build_context(fstx_ctx *ctx) {
     }
     if (rc == 0) rc = fstx_dev::event_create(&ctx->order_event);
     const uint64_t t_streams = now_ns();
-    placer.join();
+    if (placer.joinable()) placer.join();
     if (rc == 0) rc = ring_rc;
     if (rc == 0) rc = spawn_rc;
     if (bound < 0) {
