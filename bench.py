@@ -14,7 +14,7 @@ bytes / wall time of the *cold* steps (page cache dropped per file with
 warm figures (files resident in the page cache) are in ``warm``.
 
 The stdout line carries the summary (under 12 KB); every figure of the run goes to
-``--detail-out`` (default ``gpurun_out/bench_detail.json``).  On the line:
+``--detail-out`` (default ``bench_out/bench_detail.json`` next to this file).  On the line:
 
 ``roofline``      the slice-extract kernel on HBM-resident Llama-2-13B-shaped
                   tensors (config C4, TP=4, all four ranks in turn), timed with
@@ -1098,7 +1098,7 @@ def main() -> None:
     ap.add_argument("--skip-c5", action="store_true", help="leave out the 72.7 GB whole load of config C5 from tmpfs")
     ap.add_argument("--kernels-only", action="store_true",
                     help="run only the HBM kernel section (short; the command the counter profiles use)")
-    ap.add_argument("--detail-out", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+    ap.add_argument("--detail-out", default=os.path.join(ROOT, "bench_out", "bench_detail.json"),
                     help="file that receives every figure of the run; the stdout line carries the summary")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
