@@ -19,7 +19,7 @@ import logging
 import os
 from collections import OrderedDict
 from dataclasses import dataclass
-from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
+from typing import Any, Dict, List, Mapping, Optional, Sequence, Tuple, Union
 
 from .st_types import Device, DType, dtype_bits
 
@@ -87,6 +87,7 @@ def _check_header_size(n: int, buffer_len: int, where: str) -> None:
 
 Index = Union[int, slice]
 _DTYPE_OF_TAG = {d.value: d for d in DType}
+_BITS_OF_TAG = {d.value: dtype_bits(d) for d in DType if d.value != "AUTO"}
 
 
 @dataclass
@@ -167,6 +168,54 @@ class TensorFrame:
         return self.data_offsets[1] - self.data_offsets[0]
 
 
+class LazyFrames(Mapping):
+    """``name -> TensorFrame`` of one file, in offset order, over the header's own entries.
+
+    The header has been validated by whoever builds this; the frame objects -- hundreds per file --
+    are made at the first look at one of them, all at once.  Keys, length and membership need none,
+    so registering a file's names costs no frame, and a loader makes them while the file's bytes
+    are already on their way."""
+
+    __slots__ = ("_entries", "_frames")
+
+    def __init__(self, entries: Dict[str, Dict[str, Any]]):
+        self._entries = entries
+        self._frames: Optional[Dict[str, TensorFrame]] = None
+
+    def _all(self) -> Dict[str, TensorFrame]:
+        if self._frames is None:
+            self._frames = {name: TensorFrame.from_buffer(entry) for name, entry in self._entries.items()}
+        return self._frames
+
+    def __getitem__(self, name: str) -> TensorFrame:
+        return self._all()[name]
+
+    def __iter__(self):
+        return iter(self._entries)
+
+    def __len__(self) -> int:
+        return len(self._entries)
+
+    def __contains__(self, name: object) -> bool:
+        return name in self._entries
+
+    def keys(self):
+        return self._entries.keys()
+
+    def values(self):
+        return self._all().values()
+
+    def items(self):
+        return self._all().items()
+
+    def spans(self) -> List[Tuple[int, int]]:
+        """(first byte in the data section, bytes) of every tensor, without making a frame."""
+        return [(e["data_offsets"][0], e["data_offsets"][1] - e["data_offsets"][0]) for e in self._entries.values()]
+
+    def __repr__(self) -> str:
+        return repr(dict(self._all()))
+
+
 class SafeTensorsMetadata:
     """Parsed and validated header of one ``.safetensors`` file."""
 
@@ -190,7 +239,6 @@ class SafeTensorsMetadata:
         ptr_align = framework.get_device_ptr_align() if framework is not None else 16
         self.aligned = header_length % ptr_align == 0
 
-        self.tensors: Dict[str, TensorFrame] = {}
         cursor = 0
         items = list(table.items())
         spans = [tuple(entry["data_offsets"]) for _, entry in items]
@@ -199,22 +247,25 @@ class SafeTensorsMetadata:
             # (the reference sorts by begin alone and then depends on the order of the JSON for such a pair)
             items.sort(key=lambda kv: tuple(kv[1]["data_offsets"]))
         for name, entry in items:
-            frame = TensorFrame.from_buffer(entry)
-            begin, end = frame.data_offsets
+            begin, end = entry["data_offsets"]
             if begin != cursor or end < begin:
                 raise Exception(
                     f"validate(tensor {name}): InvalidOffset s={begin}, start={cursor}, e={end}, src={src}"
                 )
             count = 1
-            for extent in frame.shape:
+            for extent in entry["shape"]:
                 count *= extent
-            expect = count * dtype_bits(frame.dtype) // 8
+            bits = _BITS_OF_TAG.get(entry["dtype"])
+            if bits is None:
+                bits = dtype_bits(DType(entry["dtype"]))  # raises for an unknown tag, as the enum does
+            expect = count * bits // 8
             if end - begin != expect:
                 raise Exception(
                     f"validate(tensor {name}): TensorInvalidInfo, e-s={end - begin}, nbytes={expect}, src={src}"
                 )
-            self.tensors[name] = frame
             cursor = end
+        # the frames themselves are made when somebody first asks for one
+        self.tensors: Mapping = LazyFrames(dict(items))
         self.data_length = cursor
         if header_length + cursor > size_bytes:
             raise Exception(

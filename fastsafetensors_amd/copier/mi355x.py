@@ -50,16 +50,18 @@ def _align_up(v: int, a: int) -> int:
     return -(-v // a) * a
 
 
-def pick_lead(frames: List[TensorFrame], align: int = PTR_ALIGN, line: int = LINE_ALIGN) -> int:
+def pick_lead(frames, align: int = PTR_ALIGN, line: int = LINE_ALIGN) -> int:
     """Offset 0..line-1 of the data section inside the arena that puts the most tensor
     bytes on an ``align`` boundary and, among those, the most on a ``line`` boundary
     (ties go to the smallest offset).  The first is what callers are promised; the second
-    lets the copy kernels run over whole cache lines."""
+    lets the copy kernels run over whole cache lines.  ``frames``: tensor frames, or
+    (first byte, bytes) pairs."""
     on_align = [0] * align
     on_line = [0] * line
     for f in frames:
-        on_align[-f.data_offsets[0] % align] += f.nbytes
-        on_line[-f.data_offsets[0] % line] += f.nbytes
+        begin, nbytes = f if isinstance(f, tuple) else (f.data_offsets[0], f.nbytes)
+        on_align[-begin % align] += nbytes
+        on_line[-begin % line] += nbytes
     return max(range(line), key=lambda lead: (on_align[lead % align], on_line[lead], -lead))
 
 
@@ -96,7 +98,7 @@ class MI355XFileCopier(CopierInterface):
             self.data_at = meta.header_length - first
         else:
             first = meta.header_length
-            self.data_at = pick_lead(list(meta.tensors.values()))
+            self.data_at = pick_lead(meta.tensors.spans())  # from the header's entries: the frames are made during the transfer
         total = meta.size_bytes - first
         lead = self.data_at if self.layout == "direct" else 0
         gbuf = self.framework.alloc_tensor_memory(lead + total, self.device)

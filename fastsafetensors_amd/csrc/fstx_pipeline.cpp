@@ -820,7 +820,7 @@ struct Worker {
         for (int pass = 0; pass < 2; ++pass) {
             const uint64_t from = pass == 0 ? 0 : head, to = pass == 0 ? head : ctx->slot_bytes;
             for (uint64_t s = index; s < slots; s += helpers) {
-                if (pass == 0 && ctx->head_mapped[s].load(std::memory_order_relaxed)) continue; // its owner has been there
+                if (pass == 0 && ctx->head_mapped[s].exchange(1, std::memory_order_relaxed)) continue; // somebody has been there, or is
                 const char *base = ctx->ring + s * ctx->slot_bytes;
                 for (uint64_t at = from; at < to; at += kPage) {
                     if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
@@ -844,6 +844,8 @@ struct Worker {
         uint64_t done = 0;
         char sink = 0;
         for (uint32_t k = 0; k < mine->size(); ++k) {
+            // whoever gets to a slot's head first maps it (another worker may be going through the whole ring)
+            if (ctx->head_mapped[(uint64_t)index * ctx->cfg.slots_per_thread + k].exchange(1, std::memory_order_relaxed)) continue;
             const char *base = (*mine)[k].host;
             for (uint64_t at = 0; at < head; at += kPage) {
                 if ((at & (16 * kPage - 1)) == 0 && ctx->parts_seen.load(std::memory_order_acquire) &&
@@ -852,7 +854,6 @@ struct Worker {
                 sink ^= *(const volatile char *)(base + at);
                 done += kPage;
             }
-            ctx->head_mapped[(uint64_t)index * ctx->cfg.slots_per_thread + k].store(1, std::memory_order_relaxed);
         }
     out:
         (void)sink;

@@ -41,7 +41,7 @@ class FilesBufferOnDevice:
             self.instantiated[rank] = {}
             for lidx, factory in enumerate(factories):
                 self.instantiated[rank][lidx] = {}
-                for key in factory.metadata.tensors:
+                for key in factory.metadata.tensors.keys():  # (names only: no frame is made for this)
                     if key in self.key_to_rank_lidx:
                         raise Exception(f"FilesBufferOnDevice: key {key} must be unique among files")
                     self.key_to_rank_lidx[key] = (rank, lidx)

@@ -34,6 +34,35 @@ logger = init_logger(__name__)
 DEFAULT_COPIER = "mi355x"
 
 
+class FramesOfFiles(Mapping):
+    """``name -> TensorFrame`` over the files registered with a loader, in registration order.
+    Holds each file's own (lazy) mapping and an index of the names; a later file's tensor replaces
+    an earlier one of the same name, as ``dict.update`` would."""
+
+    def __init__(self) -> None:
+        self._files: List[Mapping] = []
+        self._where: Dict[str, int] = {}
+
+    def add(self, frames: Mapping) -> None:
+        self._where.update(dict.fromkeys(frames.keys(), len(self._files)))
+        self._files.append(frames)
+
+    def __getitem__(self, name: str) -> TensorFrame:
+        return self._files[self._where[name]][name]
+
+    def __iter__(self):
+        return iter(self._where)
+
+    def __len__(self) -> int:
+        return len(self._where)
+
+    def __contains__(self, name: object) -> bool:
+        return name in self._where
+
+    def keys(self):
+        return self._where.keys()
+
+
 class BaseSafeTensorsFileLoader:
     """Loader over a named copier backend; see ``SafeTensorsFileLoader`` for the usual entry."""
 
@@ -55,7 +84,7 @@ class BaseSafeTensorsFileLoader:
         self.pg = self.framework.get_process_group(pg)
         self.device = device
         self.meta: Dict[str, Tuple[SafeTensorsMetadata, int]] = {}
-        self.frames: "OrderedDict[str, TensorFrame]" = OrderedDict()
+        self.frames = FramesOfFiles()
         self.disable_cache = disable_cache
         # headers parsed ahead of add_filenames (ParallelLoader reads the next batch's while this one loads)
         self.parsed_ahead: Dict[str, SafeTensorsMetadata] = {}
@@ -66,7 +95,7 @@ class BaseSafeTensorsFileLoader:
         )
 
     def reset(self) -> None:
-        self.frames = OrderedDict()
+        self.frames = FramesOfFiles()
         self.meta = {}
 
     def close(self) -> None:
@@ -101,7 +130,7 @@ class BaseSafeTensorsFileLoader:
                 path = paths[turn]
                 metadata = self.parsed_ahead.pop(path, None) or SafeTensorsMetadata.from_file(path, self.framework)
                 self.meta[path] = (metadata, rank)
-                self.frames.update(metadata.tensors)
+                self.frames.add(metadata.tensors)
                 if rank == self.pg.rank():
                     logger.debug("add_filenames %d: path=%s", len(self.meta), path)
 

@@ -171,13 +171,13 @@ def _native_code(name: str) -> int:
 
 def test_context_built_behind_the_callers_back(sim, blob):
     """FSTX_CREATE_ASYNC: create returns before ring, streams and workers exist (here the pinned
-    allocation takes 150 ms); files are opened and reads queued meanwhile, and the wait delivers
+    allocation takes 400 ms); files are opened and reads queued meanwhile, and the wait delivers
     the bytes once the build is through.  The same configuration without the flag names the same
     shared context."""
     path, data = blob
     import time
 
-    sim.fstx_sim_set_host_alloc_delay_us(150_000)
+    sim.fstx_sim_set_host_alloc_delay_us(400_000)
     try:
         t0 = time.perf_counter()
         ctx = make_ctx(sim, block=64 * 1024, flags=_native.CREATE_ASYNC)
@@ -185,12 +185,12 @@ def test_context_built_behind_the_callers_back(sim, blob):
         dev = np.zeros(data.size, dtype=np.uint8)
         req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
         queued_after = time.perf_counter() - t0
-        assert req >= 1 and queued_after < 0.1, queued_after  # nothing waited for the build
+        assert req >= 1 and queued_after < 0.3, queued_after  # nothing waited for the build
         assert sim.fstx_wait_read(ctx, req) == data.size
-        assert time.perf_counter() - t0 >= 0.15
+        assert time.perf_counter() - t0 >= 0.4
         assert np.array_equal(dev, data)
         m = metrics(sim, ctx)
-        assert m.create_ns >= 150_000_000 and m.bytes_copied == data.size
+        assert m.create_ns >= 400_000_000 and m.bytes_copied == data.size
         assert sim.fstx_file_close(ctx, f) == 0
         # destroying a context right after asking for it waits for the build, then takes it apart
         other = make_ctx(sim, block=8192, flags=_native.CREATE_ASYNC)

@@ -358,6 +358,26 @@ def big_file(tmp_path_factory):
     return path, data
 
 
+def timing_test(attempts=3):
+    """A test of a controller that steers by measured rates: on a machine whose CPUs come and go
+    (a shared virtual machine) one run can be starved into a wrong reading, so the property must
+    hold in one of a few attempts; what fails every time is reported."""
+    def wrap(fn):
+        import functools
+
+        @functools.wraps(fn)
+        def run(*args, **kwargs):
+            for attempt in range(attempts):
+                try:
+                    return fn(*args, **kwargs)
+                except AssertionError:
+                    if attempt + 1 == attempts:
+                        raise
+        return run
+    return wrap
+
+
+@timing_test()
 def test_depth_climbs_on_parallel_storage_and_stays_low_on_serial_storage(sim, big_file):
     """Model: a request of 64 KiB takes 5 ms + 64 KiB at bandwidth / parallel (another 5 ms); up to
     `parallel` requests are served at once.  (Slow on purpose: the model, not this machine's
@@ -378,6 +398,7 @@ def test_depth_climbs_on_parallel_storage_and_stays_low_on_serial_storage(sim, b
     assert parallel_rate > 3 * (10 * MIB / wall), (parallel_rate, 10 * MIB / wall)
 
 
+@timing_test()
 def test_staging_copies_keep_up_with_fast_storage(sim, big_file):
     """Storage modelled at 8 GB/s over 8 channels, 4 MiB reads, depth 8: moving the bytes from the
     staging buffers into the ring is spread over all workers, and they spend well under half of
