@@ -245,6 +245,7 @@ struct Request {
     int64_t id = 0;
     std::shared_ptr<FileEntry> file;
     uint64_t length = 0;
+    bool small = false; // under kSmallRequest: short blocks, few slots
     std::atomic<uint64_t> blocks_left{0};
     std::atomic<int64_t> error{0};      // first negative status seen by a worker
     std::atomic<uint64_t> stream_mask{0}; // copy streams that carry blocks of this request
@@ -459,6 +460,7 @@ struct fstx_ctx {
     uint64_t create_t0 = 0;
     uint64_t small_block = 0;     // block size for requests under kSmallRequest
     uint32_t small_workers = 0;   // workers such a request wakes on an idle context
+    uint32_t small_slots = 1;     // slots of each worker such a request goes through
     int64_t failed = 0;           // build failure, reported by every submit from then on (q_mutex)
 
     // fstx_ctx_order_after: one event, recorded on the caller's stream, awaited by the copy streams
@@ -590,10 +592,14 @@ struct Worker {
         return hook >= 0 && ctx->fault_after.fetch_sub(1) == 0;
     }
 
-    // next ring slot of this worker, its previous copy finished
-    int64_t take_slot(Slot **out) {
+    // next ring slot of this worker, its previous copy finished.  A small request stays within
+    // the first few slots: every slot it uses has pages to be mapped first, and a worker whose
+    // one copy is in flight is covered by the other workers' reads.
+    int64_t take_slot(Slot **out, bool small) {
+        const uint32_t n = small ? std::min<uint32_t>(ctx->small_slots, (uint32_t)mine->size()) : (uint32_t)mine->size();
+        if (turn >= n) turn = 0;
         Slot &slot = (*mine)[turn];
-        turn = (turn + 1) % mine->size();
+        turn = (turn + 1) % n;
         int64_t status = 0;
         if (slot.pending) {
             if (fstx_dev::event_ready(slot.ev) != 1) {
@@ -635,7 +641,7 @@ struct Worker {
     int64_t do_buffered(const Block &b) {
         if (fault_hook()) return -EIO;
         Slot *slot = nullptr;
-        int64_t status = take_slot(&slot);
+        int64_t status = take_slot(&slot, b.req->small);
         if (status < 0) return status;
         const uint64_t at = b.file_off % kPage;
         uint64_t t0 = now_ns();
@@ -726,7 +732,7 @@ struct Worker {
         if (status == 0 && ctx->no_copy) { // measuring the reads alone: the bytes stay where the read left them
             ctx->ctr.blocks_direct.fetch_add(1, std::memory_order_relaxed);
             ctx->ctr.bytes_read.fetch_add(b.len, std::memory_order_relaxed);
-        } else if (status == 0 && (status = take_slot(&slot)) == 0) {
+        } else if (status == 0 && (status = take_slot(&slot, b.req->small)) == 0) {
             uint64_t t0 = now_ns();
             std::memcpy(slot->host, st.bytes, b.len);
             ctx->ctr.stage_ns.fetch_add(now_ns() - t0, std::memory_order_relaxed);
@@ -817,21 +823,25 @@ struct Worker {
         const uint64_t head = std::min(ctx->slot_bytes, ctx->small_block + kPage);
         uint64_t done = 0;
         char sink = 0;
-        for (int pass = 0; pass < 2; ++pass) {
-            const uint64_t from = pass == 0 ? 0 : head, to = pass == 0 ? head : ctx->slot_bytes;
-            for (uint64_t s = index; s < slots; s += helpers) {
-                if (pass == 0 && ctx->head_mapped[s].exchange(1, std::memory_order_relaxed)) continue; // somebody has been there, or is
-                const char *base = ctx->ring + s * ctx->slot_bytes;
-                for (uint64_t at = from; at < to; at += kPage) {
-                    if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) {
-                        ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
-                        return;
-                    }
-                    sink ^= *(const volatile char *)(base + at);
-                    done += kPage;
-                }
+        const uint32_t per = ctx->cfg.slots_per_thread, few = std::min(ctx->small_slots, per);
+        auto touch = [&](uint64_t s, uint64_t from, uint64_t to) { // false: work has arrived
+            const char *base = ctx->ring + s * ctx->slot_bytes;
+            for (uint64_t at = from; at < to; at += kPage) {
+                if ((at & (16 * kPage - 1)) == 0 && ctx->work_seen.load(std::memory_order_acquire)) return false;
+                sink ^= *(const volatile char *)(base + at);
+                done += kPage;
             }
+            return true;
+        };
+        bool go_on = true;
+        // first the heads of the slots a small request goes through, dealt out evenly ...
+        for (uint64_t i = index; go_on && i < (uint64_t)ctx->cfg.n_threads * few; i += helpers) {
+            const uint64_t s = i / few * per + i % few;
+            if (ctx->head_mapped[s].exchange(1, std::memory_order_relaxed)) continue; // somebody has been there, or is
+            go_on = touch(s, 0, head);
         }
+        // ... then all the rest
+        for (uint64_t s = index; go_on && s < slots; s += helpers) go_on = touch(s, s % per < few ? head : 0, ctx->slot_bytes);
         (void)sink;
         ctx->ctr.pretouched_bytes.fetch_add(done, std::memory_order_relaxed);
     }
@@ -843,7 +853,7 @@ struct Worker {
         const uint64_t head = std::min(ctx->slot_bytes, ctx->small_block + kPage);
         uint64_t done = 0;
         char sink = 0;
-        for (uint32_t k = 0; k < mine->size(); ++k) {
+        for (uint32_t k = 0; k < mine->size() && k < ctx->small_slots; ++k) {
             // whoever gets to a slot's head first maps it (another worker may be going through the whole ring)
             if (ctx->head_mapped[(uint64_t)index * ctx->cfg.slots_per_thread + k].exchange(1, std::memory_order_relaxed)) continue;
             const char *base = (*mine)[k].host;
@@ -1446,10 +1456,16 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
         if (kb >= 64 && kb % 4 == 0) ctx->small_block = kb * 1024;
     }
 
-    ctx->small_workers = std::min(cfg.n_threads, std::max(4u, cfg.n_threads / 2));
+    // measured on 0.5 and 0.7 GB files in the page cache: twelve workers with one slot each beat
+    // eight with two by 4 to 6 % (12 MiB of pinned memory to map before the link runs, not 16)
+    ctx->small_workers = std::min(cfg.n_threads, std::max(4u, cfg.n_threads * 3 / 4));
     if (const char *e = std::getenv("FSTX_SMALL_WORKERS")) {
         const uint64_t n = std::strtoull(e, nullptr, 10);
         if (n >= 1) ctx->small_workers = (uint32_t)std::min<uint64_t>(n, cfg.n_threads);
+    }
+    if (const char *e = std::getenv("FSTX_SMALL_SLOTS")) {
+        const uint64_t n = std::strtoull(e, nullptr, 10);
+        if (n >= 1) ctx->small_slots = (uint32_t)std::min<uint64_t>(n, cfg.slots_per_thread);
     }
     // each slot holds one block plus the 4 KiB lead-in of an unaligned start
     ctx->slot_bytes = cfg.block_bytes + kPage;
@@ -1635,6 +1651,7 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
         req->file->open_requests.fetch_add(1);
     }
     req->length = length;
+    req->small = length < kSmallRequest;
     if (file_off > req->file->size || length > req->file->size - file_off)
         req->error.store(-FSTX_E_SHORT_READ); // reported by wait_read, like a failed read
 
@@ -1667,7 +1684,8 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
             }
             const bool idle = ctx->queue.empty() && ctx->staged.empty();
             const uint32_t all = ctx->cfg.n_threads;
-            ctx->active_workers = idle && length < kSmallRequest ? ctx->small_workers : all;
+            // (and no more of them than there are blocks: the others would wake to find nothing)
+            ctx->active_workers = idle && req->small ? (uint32_t)std::min<uint64_t>(ctx->small_workers, blocks.size()) : all;
             for (Block &b : blocks) {
                 ctx->queue_bytes += b.len;
                 ctx->queue.push_back(std::move(b));
