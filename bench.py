@@ -340,7 +340,9 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, wi
     = 2 mod 8) -- the sizes of the reference's published single-file figures
     (docs/amd-perf.md:72-86) -- cold and warm, loader construction to last tensor.  For a file
     this small the fixed costs show: building the reader, and mapping the pages of the freshly
-    pinned ring at their first touch.  ``warm_held_reader`` is the same load while the process
+    pinned ring at their first touch -- which only the first load of a process pays, since a closed
+    reader leaves its ring parked for the next one (``warm_fresh_ring``: the same with that switched
+    off, for loads and legs alike).  ``warm_held_reader`` is the same load while the process
     keeps its reader (``hold_reader``), as a server that loads many small files would.  C2 also
     runs in the window layout, where every tensor goes through the realign kernel."""
     import torch
@@ -396,6 +398,25 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, wi
     co = max(legs, key=lambda r: r["GBps"])
     for k in variants:
         out[k] = best(lambda it=iter(loads[k]): next(it), reps=len(loads[k]))
+    # the same with nothing left behind by an earlier load: every reader allocates its pinned ring and
+    # maps its pages at their first touch, as the first load of a process does
+    from fastsafetensors_amd import release_cached_memory
+
+    parked_before = os.environ.get("FSTX_RING_CACHE")
+    os.environ["FSTX_RING_CACHE"] = "0"
+    release_cached_memory()
+    try:
+        fresh_loads, fresh_legs = [], []
+        for _ in range(4):
+            fresh_legs.append(leg("copy_only", False, reps=2))
+            fresh_loads += [run_load(files, "auto", threads, 4096, None) for _ in range(2)]
+        co_fresh = max(fresh_legs, key=lambda r: r["GBps"])
+        out["warm_fresh_ring"] = best(lambda it=iter(fresh_loads): next(it), reps=len(fresh_loads))
+    finally:
+        if parked_before is None:
+            os.environ.pop("FSTX_RING_CACHE", None)
+        else:
+            os.environ["FSTX_RING_CACHE"] = parked_before
     hold = hold_reader("cuda:0", max_threads=threads, block_size_kb=4096)
     try:
         run_load(files, "auto", threads, 4096, None)  # maps the ring's pages
@@ -407,10 +428,10 @@ def bench_small_checkpoint(key: str, data_dir: str, threads: int, write=None, wi
         out["warm_held_reader"] = best(lambda it=iter(held_loads): next(it), reps=len(held_loads))
     finally:
         hold.close()
-    for k in ("warm", "warm_held_reader", "warm_window_layout_realign"):
+    for k in ("warm", "warm_fresh_ring", "warm_held_reader", "warm_window_layout_realign"):
         if k in out:
             # a load under a held reader is compared with the leg of an engine that existed before, too
-            ceiling = co_held if k == "warm_held_reader" else co
+            ceiling = {"warm_held_reader": co_held, "warm_fresh_ring": co_fresh}.get(k, co)
             out[k]["copy_only_leg_GBps"] = ceiling["GBps"]
             out[k]["frac_of_copy_only_leg"] = out[k]["GBps"] / ceiling["GBps"]
     if with_cpu:
@@ -1243,7 +1264,8 @@ def main() -> None:
             small[k] = bench_small_checkpoint(k, os.path.join(args.dir, k + "_small"), args.threads, write, with_cpu=not args.skip_cpu_baseline)
             w = small[k]["warm"]
             log(f"[bench] {k}: cold {small[k]['cold']['GBps']:.2f} GB/s (io {small[k]['cold']['io_over_read_only_leg']:.3f} x read-only leg), "
-                f"warm {w['GBps']:.1f} GB/s = {w['frac_of_copy_only_leg']:.3f} of the copy-only leg, held "
+                f"warm {w['GBps']:.1f} GB/s = {w['frac_of_copy_only_leg']:.3f} of the copy-only leg "
+                f"(no ring left parked by an earlier load: {small[k]['warm_fresh_ring']['frac_of_copy_only_leg']:.3f}), held "
                 f"{small[k]['warm_held_reader']['frac_of_copy_only_leg']:.3f}"
                 + (f", window layout {small[k]['warm_window_layout_realign']['frac_of_copy_only_leg']:.3f}" if k == "C2" else ""))
         # ---- C4: whole load from tmpfs, then the tensor-parallel callers over the resident checkpoint
@@ -1433,6 +1455,8 @@ def main() -> None:
                "cold_io_over_read_only_leg": r3(sc["cold"]["io_over_read_only_leg"]),
                "warm_GBps": r3(sc["warm"]["GBps"]), "warm_s": round(sc["warm"]["seconds"], 4),
                "warm_frac_of_copy_only_leg": r3(sc["warm"]["frac_of_copy_only_leg"]),
+               "warm_fresh_ring_GBps": r3(sc["warm_fresh_ring"]["GBps"]),  # FSTX_RING_CACHE=0: as the first load of a process
+               "warm_fresh_ring_frac": r3(sc["warm_fresh_ring"]["frac_of_copy_only_leg"]),
                "warm_held_reader_GBps": r3(sc["warm_held_reader"]["GBps"]),
                "warm_held_reader_frac": r3(sc["warm_held_reader"]["frac_of_copy_only_leg"])}
         if "cpu_reference" in sc:

@@ -3,6 +3,7 @@
 
 __version__ = "0.1.0"
 
+from ._native import trim_cache as release_cached_memory
 from .copier.mi355x import hold_reader
 from .common import SafeTensorsMetadata, SingleGroup, TensorFrame, get_device_numa_node
 from .file_buffer import FilesBufferOnDevice
@@ -27,4 +28,5 @@ __all__ = [
     "fastsafe_open",
     "get_device_numa_node",
     "hold_reader",
+    "release_cached_memory",
 ]

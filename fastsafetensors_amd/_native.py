@@ -18,7 +18,7 @@ _LIB_NAME = "libfstx.so"
 _lib: Optional[ctypes.CDLL] = None
 _lib_lock = threading.Lock()
 
-FSTX_ABI_VERSION = 3
+FSTX_ABI_VERSION = 4
 FSTX_BATCH_MAX = 48
 READ_AUTO, READ_BUFFERED, READ_DIRECT = 0, 1, 2
 ADAPTIVE_DEPTH = 1
@@ -85,6 +85,7 @@ class FstxMetrics(ctypes.Structure):
             "storage_nr_requests",
             "storage_max_sectors_kb",
             "storage_flags",
+            "ring_reused",
         )
     ]
 
@@ -166,6 +167,8 @@ _SIGNATURES = {
     "fstx_node_cpus": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.c_int]),
     "fstx_set_debug_log": (None, [ctypes.c_int]),
     "fstx_bounce_buffer_bytes": (ctypes.c_uint64, []),
+    "fstx_cached_ring_bytes": (ctypes.c_uint64, []),
+    "fstx_trim_cache": (ctypes.c_uint64, []),
     "fstx_strerror": (ctypes.c_char_p, [ctypes.c_int64]),
     "fstx_host_alloc": (ctypes.c_void_p, [ctypes.c_uint64]),
     "fstx_host_free": (None, [ctypes.c_void_p]),
@@ -288,6 +291,16 @@ def node_cpus(node: int) -> List[int]:
 
 def bounce_buffer_bytes() -> int:
     return int(lib().fstx_bounce_buffer_bytes())
+
+
+def cached_ring_bytes() -> int:
+    """Bytes of the pinned ring the last closed reader left parked for the next one (0: none)."""
+    return int(lib().fstx_cached_ring_bytes())
+
+
+def trim_cache() -> int:
+    """Free the parked ring; returns the bytes freed."""
+    return int(lib().fstx_trim_cache())
 
 
 def read_buffer(addr: int, length: int) -> bytes:

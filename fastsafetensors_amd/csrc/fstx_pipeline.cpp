@@ -279,6 +279,7 @@ struct Slot {
     char *host = nullptr;
     fstx_dev::event_t ev = nullptr;
     bool pending = false; // an async copy out of this slot may still be running
+    bool used = false;    // a read has written to it: its first pages are mapped
 };
 
 // Bounds the O_DIRECT preads in flight.  Storage differs a lot in the queue depth
@@ -482,6 +483,7 @@ struct fstx_ctx {
     bool shape_settled = false;
     StorageFacts storage;
     int ring_node = -1;        // node of the ring's first page, where the kernel says (ready_mutex)
+    bool ring_reused = false;  // the ring is the one an earlier context of this process left behind
     uint64_t direct_bytes = 0; // bytes one O_DIRECT pread may cover
     // ordinary page-backed blocks that O_DIRECT reads land in; handed out together
     // with the read token (under q_mutex), returned after the last byte left for the ring
@@ -600,6 +602,7 @@ struct Worker {
         if (turn >= n) turn = 0;
         Slot &slot = (*mine)[turn];
         turn = (turn + 1) % n;
+        slot.used = true;
         int64_t status = 0;
         if (slot.pending) {
             if (fstx_dev::event_ready(slot.ev) != 1) {
@@ -1195,6 +1198,60 @@ int normalize(fstx_config &cfg) {
     return 0;
 }
 
+// The ring of the context that was destroyed last stays allocated for the next context of the
+// same device, node and size in this process: a fresh ring costs its allocation (0.2 to 0.5 ms)
+// and, far more, the mapping of every page at its first touch (1 ms per 12 MiB with twelve
+// threads at it), which is a tenth of the time a 0.5 GB file takes to load.  One ring at most;
+// fstx_trim_cache frees it, FSTX_RING_CACHE=0 keeps the library from parking any.
+struct ParkedRing {
+    void *p = nullptr;
+    uint64_t bytes = 0;
+    int device = -1, node = -1, ring_node = -1;
+    std::vector<uint8_t> head_mapped; // per slot: its first pages have been touched
+};
+std::mutex g_park_mutex;
+ParkedRing g_parked;
+
+bool ring_cache_on() {
+    const char *e = std::getenv("FSTX_RING_CACHE");
+    return !(e && e[0] == '0');
+}
+
+// the parked ring, if it fits; the caller owns it from here on
+bool take_parked(int device, int node, uint64_t bytes, ParkedRing &out) {
+    if (!ring_cache_on()) return false;
+    std::lock_guard<std::mutex> lk(g_park_mutex);
+    if (!g_parked.p || g_parked.device != device || g_parked.node != node || g_parked.bytes != bytes) return false;
+    out = std::move(g_parked);
+    g_parked = ParkedRing{};
+    return true;
+}
+
+// leaves the ring of a context behind for the next one (replacing what is parked), or frees it
+void park_or_free_ring(fstx_ctx *ctx) {
+    ParkedRing old;
+    if (ring_cache_on() && ctx->build_status == 0 && !ctx->failed) {
+        ParkedRing mine;
+        mine.p = ctx->ring;
+        mine.bytes = ctx->ring_bytes;
+        mine.device = ctx->cfg.device_id;
+        mine.node = ctx->cfg.numa_node;
+        mine.ring_node = ctx->ring_node;
+        const uint32_t per = ctx->cfg.slots_per_thread;
+        mine.head_mapped.resize((size_t)ctx->cfg.n_threads * per);
+        for (uint32_t w = 0; w < ctx->cfg.n_threads; ++w)
+            for (uint32_t k = 0; k < per; ++k)
+                mine.head_mapped[(size_t)w * per + k] =
+                    ctx->head_mapped[(size_t)w * per + k].load() || (k < ctx->slots[w].size() && ctx->slots[w][k].used);
+        std::lock_guard<std::mutex> lk(g_park_mutex);
+        old = std::move(g_parked);
+        g_parked = std::move(mine);
+    } else {
+        old.p = ctx->ring;
+    }
+    if (old.p) fstx_dev::host_free(old.p);
+}
+
 void free_parts(fstx_ctx *ctx) {
     const uint64_t t0 = now_ns();
     for (auto &per : ctx->slots)
@@ -1206,8 +1263,8 @@ void free_parts(fstx_ctx *ctx) {
     for (auto s : ctx->streams) fstx_dev::stream_destroy(s);
     const uint64_t t2 = now_ns();
     if (ctx->ring) {
-        fstx_dev::host_free(ctx->ring);
-        fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes);
+        park_or_free_ring(ctx);
+        fstx_internal::note_bounce_bytes(-(int64_t)ctx->ring_bytes); // a parked ring is nobody's bounce buffer
     }
     fstx_internal::debug("free_parts: events %.2f ms, streams %.2f ms, ring %.2f ms", (t1 - t0) / 1e6, (t2 - t1) / 1e6,
                          (now_ns() - t2) / 1e6);
@@ -1302,12 +1359,22 @@ int build_context(fstx_ctx *ctx) {
                                (unsigned long long)(ctx->ring_bytes >> 20));
     void *p = nullptr;
     int ring_rc = 0, bound = 0, ring_node = -1;
+    bool reused = false;
     uint64_t t_ring = 0;
     auto place_ring = [&](bool own_thread) {
         if (own_thread) bound = bind_thread_to_node(cfg.numa_node); // never the caller's own affinity and policy
         ring_rc = fstx_dev::set_device(cfg.device_id);
-        if (ring_rc == 0) ring_rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
-        if (ring_rc == 0 && p && cfg.numa_node >= 0) {
+        ParkedRing parked;
+        if (ring_rc == 0 && take_parked(cfg.device_id, cfg.numa_node, ctx->ring_bytes, parked)) {
+            // the ring an earlier context left behind: allocated, placed, and mapped where it was used
+            p = parked.p;
+            ring_node = parked.ring_node;
+            reused = true;
+            for (size_t i = 0; i < parked.head_mapped.size(); ++i)
+                if (parked.head_mapped[i]) ctx->head_mapped[i].store(1, std::memory_order_relaxed);
+        }
+        if (ring_rc == 0 && !p) ring_rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
+        if (ring_rc == 0 && p && !reused && cfg.numa_node >= 0) {
             *static_cast<volatile char *>(p) = 0; // the page exists from here on, on the node the policy names
             ring_node = node_of_address(p);
         }
@@ -1322,6 +1389,7 @@ int build_context(fstx_ctx *ctx) {
                 ctx->parts_status = ring_rc ? ring_rc : -FSTX_E_HIP;
             }
             ctx->ring_node = ring_node;
+            ctx->ring_reused = reused;
             ctx->ring_ready = true;
         }
         ctx->ready_cv.notify_all();
@@ -1428,6 +1496,23 @@ void teardown(fstx_ctx *ctx) {
 }
 
 } // namespace
+
+uint64_t fstx_cached_ring_bytes(void) {
+    std::lock_guard<std::mutex> lk(g_park_mutex);
+    return g_parked.p ? g_parked.bytes : 0;
+}
+
+uint64_t fstx_trim_cache(void) {
+    ParkedRing old;
+    {
+        std::lock_guard<std::mutex> lk(g_park_mutex);
+        old = std::move(g_parked);
+        g_parked = ParkedRing{};
+    }
+    if (!old.p) return 0;
+    fstx_dev::host_free(old.p);
+    return old.bytes;
+}
 
 int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (!cfg_in || !out || cfg_in->struct_size < sizeof(fstx_config)) return -FSTX_E_INVAL;
@@ -1803,6 +1888,7 @@ int fstx_get_metrics(fstx_ctx *ctx, fstx_metrics *out) {
     m.bind_errors = c.bind_errors.load();
     m.first_bind_error = c.first_bind_error.load();
     m.pretouched_bytes = c.pretouched_bytes.load();
+    m.ring_reused = ctx->ring_reused ? 1 : 0;
     {
         std::lock_guard<std::mutex> lk(ctx->q_mutex);
         m.direct_read_bytes = ctx->shape_settled ? ctx->direct_bytes : 0;

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FSTX_ABI_VERSION 3
+#define FSTX_ABI_VERSION 4
 
 /* status codes beyond errno */
 #define FSTX_E_BASE 10000
@@ -148,6 +148,7 @@ typedef struct fstx_metrics {
     uint64_t storage_nr_requests; /* /sys/dev/block/<dev>/queue/nr_requests of that file's device */
     uint64_t storage_max_sectors_kb;
     uint64_t storage_flags;       /* FSTX_STORAGE_*                                              */
+    uint64_t ring_reused;         /* 1 = the ring is the one the last destroyed context left parked */
 } fstx_metrics;
 
 /* ---- library-wide helpers ------------------------------------------------ */
@@ -182,9 +183,20 @@ int fstx_node_cpus(int numa_node, int *cpus, int capacity);
 /* Toggle debug lines on stderr.  set_debug_log (cpp/ext.cpp:417-420). */
 void fstx_set_debug_log(int enabled);
 
-/* Pinned ring bytes alive in the whole process.
+/* Pinned ring bytes of all contexts alive in the process (a parked ring belongs to none).
  * get_cpp_metrics().bounce_buffer_bytes (cpp/ext.cpp:952-954). */
 uint64_t fstx_bounce_buffer_bytes(void);
+
+/* The pinned ring of the context that was destroyed last stays allocated ("parked") for the next
+ * context of the same device, node and ring size in this process, which thereby skips the
+ * allocation and, above all, the page-by-page mapping of fresh pinned memory at its first touch
+ * (the reference allocates its bounce buffer per reader, nogds.py:107-116 / ext.cpp:648-672, and
+ * pays that every time).  At most one ring is parked; it is not counted by
+ * fstx_bounce_buffer_bytes.  fstx_cached_ring_bytes tells its size, fstx_trim_cache frees it
+ * (returns the bytes freed); with FSTX_RING_CACHE=0 in the environment nothing is ever parked.
+ * No counterpart in the reference. */
+uint64_t fstx_cached_ring_bytes(void);
+uint64_t fstx_trim_cache(void);
 
 /* Text for a negative return value (errno or fstx_status); never NULL. */
 const char *fstx_strerror(int64_t code);

@@ -107,8 +107,19 @@ int main(int argc, char **argv) {
         int cpus[4];
         CHECK(fstx_node_cpus(-1, cpus, 4) < 0);
     }
+    const uint64_t ring_of_ctx = met.bounce_buffer_bytes;
     CHECK(fstx_ctx_destroy(ctx) == 0);
     CHECK(fstx_bounce_buffer_bytes() == 0);
+    /* the ring stays parked for the next context of this shape, which takes it over; trimming frees it */
+    CHECK(fstx_cached_ring_bytes() == ring_of_ctx);
+    {
+        fstx_ctx *next = NULL;
+        CHECK(fstx_ctx_create(&cfg, &next) == 0);
+        met.struct_size = sizeof met;
+        CHECK(fstx_get_metrics(next, &met) == 0 && met.ring_reused == 1 && fstx_cached_ring_bytes() == 0);
+        CHECK(fstx_ctx_destroy(next) == 0 && fstx_cached_ring_bytes() == ring_of_ctx);
+        CHECK(fstx_trim_cache() == ring_of_ctx && fstx_cached_ring_bytes() == 0 && fstx_trim_cache() == 0);
+    }
 
     /* ---- a shared context: two users, one ring; ordered after the null stream's work ---- */
     {

@@ -44,8 +44,11 @@ int main(int argc, char **argv) {
         close(fd);
     }
     fstx_sim_set_copy_delay_us(20);
+    const char *cache_env = std::getenv("FSTX_RING_CACHE");
+    const bool ring_cache_expected = !(cache_env && cache_env[0] == '0');
     std::atomic<int> bad{0};
-    for (int round = 0; round < rounds; ++round) {
+    for (int turn = 0; turn < 2 * rounds; ++turn) {
+        const int round = turn / 2; // every shape twice in a row: the second context takes over the ring the first left parked
         fstx_config cfg{};
         cfg.struct_size = sizeof cfg;
         cfg.device_id = 0;
@@ -101,11 +104,13 @@ int main(int argc, char **argv) {
         m.struct_size = sizeof m;
         fstx_get_metrics(ctx, &m);
         if (m.bytes_copied != 3 * size) bad++;
+        if (ring_cache_expected && m.ring_reused != (uint64_t)(turn % 2)) bad++;
         fstx_sim_stream_destroy(foreign); // drains it: the stand-in's events must outlive their records
         if (again && fstx_ctx_release(again) != 0) bad++;
         if ((again ? fstx_ctx_release(ctx) : fstx_ctx_destroy(ctx)) != 0) bad++;
     }
-    if (fstx_bounce_buffer_bytes() != 0) bad++;
+    fstx_trim_cache(); // the ring the last context left parked
+    if (fstx_bounce_buffer_bytes() != 0 || fstx_cached_ring_bytes() != 0) bad++;
     std::printf("hostsim_driver: %s\n", bad.load() ? "MISMATCH" : "ok");
     return bad.load() ? 1 : 0;
 }

@@ -26,14 +26,14 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(_native.library_path())
     for name in declared_functions():
         assert hasattr(raw, name), name
-    assert _native.lib().fstx_abi_version() == _native.FSTX_ABI_VERSION == 3
+    assert _native.lib().fstx_abi_version() == _native.FSTX_ABI_VERSION == 4
 
 
 def test_constants_match_the_header():
     text = open(os.path.join(ROOT, "include", "fstx.h")).read()
     assert int(re.search(r"#define FSTX_BATCH_MAX (\d+)", text).group(1)) == _native.FSTX_BATCH_MAX
     assert int(re.search(r"#define FSTX_ABI_VERSION (\d+)", text).group(1)) == _native.FSTX_ABI_VERSION
-    assert ctypes.sizeof(_native.FstxConfig) == 56 and ctypes.sizeof(_native.FstxMetrics) == 200
+    assert ctypes.sizeof(_native.FstxConfig) == 56 and ctypes.sizeof(_native.FstxMetrics) == 208
     assert ctypes.sizeof(_native.FstxCopyDesc) == 24 and ctypes.sizeof(_native.FstxSliceDesc) == 40
 
 

@@ -25,6 +25,9 @@ PIPELINE_SYMBOLS = [
 
 @pytest.fixture(scope="module")
 def sim():
+    # the tests count pinned allocations: no ring stays parked between contexts unless a test asks for it
+    parked_before = os.environ.get("FSTX_RING_CACHE")
+    os.environ["FSTX_RING_CACHE"] = "0"
     if not os.path.exists(os.path.join(SIM_DIR, "libfstx_hostsim.so")):
         subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
     lib = ctypes.CDLL(os.path.join(SIM_DIR, "libfstx_hostsim.so"))
@@ -41,7 +44,12 @@ def sim():
     lib.fstx_sim_set_host_alloc_delay_us.argtypes = [ctypes.c_int]
     lib.fstx_sim_fail_host_allocs.argtypes = [ctypes.c_int]
     lib.fstx_sim_set_copy_delay_us(30)
-    return lib
+    yield lib
+    lib.fstx_trim_cache()
+    if parked_before is None:
+        os.environ.pop("FSTX_RING_CACHE", None)
+    else:
+        os.environ["FSTX_RING_CACHE"] = parked_before
 
 
 @pytest.fixture(scope="module")
@@ -548,7 +556,68 @@ def test_pipeline_under_sanitizers(blob, binary):
     if not os.path.exists(exe):
         subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
     path, _ = blob
-    run = subprocess.run([exe, path, "3"], capture_output=True, text=True, timeout=300)
+    # every shape twice in a row, so that the second context of a shape takes over the first one's ring
+    run = subprocess.run([exe, path, "3"], capture_output=True, text=True, timeout=300, env=dict(os.environ, FSTX_RING_CACHE="1"))
     assert run.returncode == 0, run.stdout + run.stderr
     assert "Sanitizer" not in run.stderr, run.stderr
     assert "hostsim_driver: ok" in run.stdout
+
+
+def test_ring_is_parked_for_the_next_context(sim, blob, monkeypatch):
+    """The ring of the context destroyed last is taken over by the next context of the same shape:
+    one allocation fewer, nothing counted as a bounce buffer meanwhile, freed by a trim, replaced by
+    the ring of a context of another shape, and never parked when the environment says no."""
+    path, data = blob
+    monkeypatch.setenv("FSTX_RING_CACHE", "1")
+    ring = lambda threads, block=64 * 1024: threads * 2 * (block + 4096)
+
+    def load(ctx):
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        dev = np.zeros(data.size, dtype=np.uint8)
+        req = sim.fstx_submit_read(ctx, f, 0, data.size, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, req) == data.size and np.array_equal(dev, data)
+        assert sim.fstx_file_close(ctx, f) == 0
+
+    a = make_ctx(sim, threads=3)
+    load(a)
+    assert metrics(sim, a).ring_reused == 0 and sim.fstx_cached_ring_bytes() == 0
+    assert sim.fstx_ctx_destroy(a) == 0
+    assert sim.fstx_bounce_buffer_bytes() == 0 and sim.fstx_sim_pinned_live() == 1
+    assert sim.fstx_cached_ring_bytes() == ring(3)
+    # same shape: taken over, also by a context that is built behind the caller's back
+    b = make_ctx(sim, threads=3, flags=_native.CREATE_ASYNC)
+    load(b)
+    assert metrics(sim, b).ring_reused == 1 and sim.fstx_cached_ring_bytes() == 0
+    assert sim.fstx_bounce_buffer_bytes() == ring(3) and sim.fstx_sim_pinned_live() == 1
+    # a second one alive at the same time gets a ring of its own; the one destroyed last stays
+    c = make_ctx(sim, threads=3)
+    assert metrics(sim, c).ring_reused == 0 and sim.fstx_sim_pinned_live() == 2
+    load(c)
+    assert sim.fstx_ctx_destroy(b) == 0 and sim.fstx_sim_pinned_live() == 2
+    assert sim.fstx_ctx_destroy(c) == 0 and sim.fstx_sim_pinned_live() == 1
+    # another shape: not taken over; its ring replaces the parked one
+    d = make_ctx(sim, threads=2)
+    assert metrics(sim, d).ring_reused == 0 and sim.fstx_sim_pinned_live() == 2
+    load(d)
+    assert sim.fstx_ctx_destroy(d) == 0
+    assert sim.fstx_sim_pinned_live() == 1 and sim.fstx_cached_ring_bytes() == ring(2)
+    assert sim.fstx_trim_cache() == ring(2) and sim.fstx_trim_cache() == 0
+    assert sim.fstx_sim_pinned_live() == 0 and sim.fstx_bounce_buffer_bytes() == 0
+    # switched off: freed with its context
+    monkeypatch.setenv("FSTX_RING_CACHE", "0")
+    e = make_ctx(sim, threads=3)
+    load(e)
+    assert sim.fstx_ctx_destroy(e) == 0
+    assert sim.fstx_sim_pinned_live() == 0 and sim.fstx_cached_ring_bytes() == 0
+
+
+def test_a_context_that_failed_parks_nothing(sim, monkeypatch):
+    monkeypatch.setenv("FSTX_RING_CACHE", "1")
+    sim.fstx_sim_fail_host_allocs(1)
+    try:
+        out = ctypes.c_void_p()
+        cfg = make_cfg(threads=3)
+        assert sim.fstx_ctx_create(ctypes.byref(cfg), ctypes.byref(out)) < 0
+        assert sim.fstx_cached_ring_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
+    finally:
+        sim.fstx_sim_fail_host_allocs(0)

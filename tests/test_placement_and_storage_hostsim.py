@@ -34,6 +34,9 @@ PIPELINE_SYMBOLS = [
 
 @pytest.fixture(scope="module")
 def sim():
+    # no ring stays parked between the contexts of these tests
+    parked_before = os.environ.get("FSTX_RING_CACHE")
+    os.environ["FSTX_RING_CACHE"] = "0"
     if not os.path.exists(os.path.join(SIM_DIR, "libfstx_hostsim.so")):
         subprocess.run(["make", "-s", "-C", SIM_DIR], check=True)
     lib = ctypes.CDLL(os.path.join(SIM_DIR, "libfstx_hostsim.so"))
@@ -47,6 +50,11 @@ def sim():
     yield lib
     lib.fstx_sim_set_storage(0, 0.0, 0)
     lib.fstx_sim_set_copy_delay_us(30)
+    lib.fstx_trim_cache()
+    if parked_before is None:
+        os.environ.pop("FSTX_RING_CACHE", None)
+    else:
+        os.environ["FSTX_RING_CACHE"] = parked_before
 
 
 class env:

@@ -175,6 +175,33 @@ def test_shared_reader_lives_as_long_as_someone_holds_it(golden):
     assert_clean()
 
 
+def test_a_closed_readers_ring_serves_the_next_reader(golden):
+    """A closed loader leaves its pinned ring parked; the next loader with the same settings takes
+    it over (no allocation, pages already mapped), loads the same bytes, and the parked ring is
+    no bounce buffer of anybody and is freed on request."""
+    import fastsafetensors_amd
+
+    path = golden("tiny_gpt2.safetensors")
+    h = orc.parse_file(path)
+    fastsafetensors_amd.release_cached_memory()
+    reused = []
+    for _ in range(3):
+        loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=3, block_size_kb=256)
+        loader.add_filenames({0: [path]})
+        bufs = loader.copy_files_to_device()
+        m = loader.copier_constructor.reader.metrics()
+        reused.append(int(m.ring_reused))
+        for name in h.tensors:
+            assert np.array_equal(dev_bytes(bufs.get_tensor(name)), orc.tensor_bytes(path, h, name)), name
+        bufs.close()
+        loader.close()
+        assert_clean()
+        assert _native.cached_ring_bytes() == m.bounce_buffer_bytes
+    assert reused == [0, 1, 1]
+    assert fastsafetensors_amd.release_cached_memory() == m.bounce_buffer_bytes
+    assert _native.cached_ring_bytes() == 0 and fastsafetensors_amd.release_cached_memory() == 0
+
+
 def test_adaptive_depth_and_small_direct_reads(tmp_path):
     """O_DIRECT with many small reads in flight and the depth steered while reading -- the
     setting for storage that wants a deep queue -- byte-exact against the oracle."""
