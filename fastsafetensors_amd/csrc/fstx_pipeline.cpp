@@ -1205,7 +1205,7 @@ int normalize(fstx_config &cfg) {
 // fstx_trim_cache frees it, FSTX_RING_CACHE=0 keeps the library from parking any.
 struct ParkedRing {
     void *p = nullptr;
-    uint64_t bytes = 0;
+    uint64_t bytes = 0, slot_bytes = 0;
     int device = -1, node = -1, ring_node = -1;
     std::vector<uint8_t> head_mapped; // per slot: its first pages have been touched
 };
@@ -1234,6 +1234,7 @@ void park_or_free_ring(fstx_ctx *ctx) {
         ParkedRing mine;
         mine.p = ctx->ring;
         mine.bytes = ctx->ring_bytes;
+        mine.slot_bytes = ctx->slot_bytes;
         mine.device = ctx->cfg.device_id;
         mine.node = ctx->cfg.numa_node;
         mine.ring_node = ctx->ring_node;
@@ -1370,8 +1371,10 @@ int build_context(fstx_ctx *ctx) {
             p = parked.p;
             ring_node = parked.ring_node;
             reused = true;
-            for (size_t i = 0; i < parked.head_mapped.size(); ++i)
-                if (parked.head_mapped[i]) ctx->head_mapped[i].store(1, std::memory_order_relaxed);
+            // (a ring of the same size cut into other slots says nothing about these)
+            if (parked.head_mapped.size() == (size_t)cfg.n_threads * cfg.slots_per_thread && parked.slot_bytes == ctx->slot_bytes)
+                for (size_t i = 0; i < parked.head_mapped.size(); ++i)
+                    if (parked.head_mapped[i]) ctx->head_mapped[i].store(1, std::memory_order_relaxed);
         }
         if (ring_rc == 0 && !p) ring_rc = fstx_dev::host_alloc(&p, ctx->ring_bytes);
         if (ring_rc == 0 && p && !reused && cfg.numa_node >= 0) {
