@@ -459,7 +459,9 @@ struct fstx_ctx {
     int build_status = 0;
     std::thread builder;          // FSTX_CREATE_ASYNC: runs build_context() behind fstx_ctx_create's back
     uint64_t create_t0 = 0;
-    uint64_t small_block = 0;     // block size for requests under kSmallRequest
+    uint64_t small_block = 0;     // block size for small requests (see fstx_submit_read) on a ring whose pages are yet to be mapped
+    uint64_t small_block_mapped = 0; // ... and on a ring that an earlier context has used
+    uint64_t burst_bytes = 0;     // bytes submitted since a submit last found nothing queued (q_mutex)
     uint32_t small_workers = 0;   // workers such a request wakes on an idle context
     uint32_t small_slots = 1;     // slots of each worker such a request goes through
     int64_t failed = 0;           // build failure, reported by every submit from then on (q_mutex)
@@ -1539,9 +1541,10 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
     if (cfg.max_direct_reads && cfg.direct_read_bytes) settle_direct_shape(ctx.get(), StorageFacts{});
     if (const char *e = std::getenv("FSTX_FAULT_READ_AFTER")) ctx->fault_after.store(std::atoll(e));
     ctx->small_block = kSmallRequestBlock;
+    ctx->small_block_mapped = 2 * kSmallRequestBlock;
     if (const char *e = std::getenv("FSTX_SMALL_BLOCK_KB")) {
         const uint64_t kb = std::strtoull(e, nullptr, 10);
-        if (kb >= 64 && kb % 4 == 0) ctx->small_block = kb * 1024;
+        if (kb >= 64 && kb % 4 == 0) ctx->small_block = ctx->small_block_mapped = kb * 1024;
     }
 
     // measured on 0.5 and 0.7 GB files in the page cache: twelve workers with one slot each beat
@@ -1739,7 +1742,16 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
         req->file->open_requests.fetch_add(1);
     }
     req->length = length;
-    req->small = length < kSmallRequest;
+    {
+        // A request is small while less than 2 GiB have been submitted since a submit last found
+        // nothing queued: a single file of that size, or the first files of a checkpoint made of
+        // many.  (Eight files of 1.9 GB each, all cut into 1 MiB blocks, load at 53.8 GB/s; with
+        // only the first of them treated so, at 56.)
+        std::lock_guard<std::mutex> lk(ctx->q_mutex);
+        if (ctx->queue.empty() && ctx->staged.empty()) ctx->burst_bytes = 0;
+        ctx->burst_bytes += length;
+        req->small = ctx->burst_bytes < kSmallRequest;
+    }
     if (file_off > req->file->size || length > req->file->size - file_off)
         req->error.store(-FSTX_E_SHORT_READ); // reported by wait_read, like a failed read
 
@@ -1747,12 +1759,23 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
     // first byte, so that every block's O_DIRECT window fits one slot.
     std::vector<Block> blocks;
     if (length && req->error.load() == 0) {
-        // Requests under 2 GiB are cut into blocks of 1 MiB: a slot's pages are mapped at their
+        // Small requests are cut into blocks of 1 MiB: a slot's pages are mapped at their
         // first touch, at 18 GB/s at best, so a load moves at that rate until the part of the ring
         // it uses has been touched once -- 2.5 ms for 32 slots of 2 MiB, which is a sixth of a
-        // 0.7 GB load.  1 MiB blocks still run the link at 56 of its 57 GB/s.
+        // 0.7 GB load.  1 MiB blocks still run the link at 54 of its 57 GB/s.  On a ring that an
+        // earlier context has left behind there is little or nothing to map: 2 MiB blocks, which
+        // run the link at 56 (0.5 and 0.7 GB files: 10.0 and 14.1 ms against 10.5 and 15.1).
         uint64_t bb = ctx->cfg.block_bytes;
-        if (length < kSmallRequest) bb = std::min(bb, ctx->small_block);
+        if (req->small) {
+            bool mapped;
+            {
+                std::lock_guard<std::mutex> lk(ctx->ready_mutex);
+                mapped = ctx->ring_ready && ctx->ring_reused; // (a ring that is still being allocated is a fresh one)
+            }
+            // (likewise the ring of a context that has served requests before: a reader that is held)
+            mapped = mapped || ctx->ctr.bytes_read.load(std::memory_order_relaxed) > 0;
+            bb = std::min(bb, mapped ? ctx->small_block_mapped : ctx->small_block);
+        }
         const uint64_t origin = align_down(file_off, kPage);
         const uint64_t end = file_off + length;
         for (uint64_t lo = origin; lo < end; lo += bb) {
