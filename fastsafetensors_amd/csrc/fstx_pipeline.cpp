@@ -462,6 +462,7 @@ struct fstx_ctx {
     uint64_t small_block = 0;     // block size for small requests (see fstx_submit_read) on a ring whose pages are yet to be mapped
     uint64_t small_block_mapped = 0; // ... and on a ring that an earlier context has used
     uint64_t burst_bytes = 0;     // bytes submitted since a submit last found nothing queued (q_mutex)
+    uint64_t small_burst = 0;     // requests are small while burst_bytes stays under this
     uint32_t small_workers = 0;   // workers such a request wakes on an idle context
     uint32_t small_slots = 1;     // slots of each worker such a request goes through
     int64_t failed = 0;           // build failure, reported by every submit from then on (q_mutex)
@@ -1549,6 +1550,11 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 
     // measured on 0.5 and 0.7 GB files in the page cache: twelve workers with one slot each beat
     // eight with two by 4 to 6 % (12 MiB of pinned memory to map before the link runs, not 16)
+    ctx->small_burst = kSmallRequest;
+    if (const char *e = std::getenv("FSTX_SMALL_BURST_MB")) {
+        const uint64_t mb = std::strtoull(e, nullptr, 10);
+        if (mb >= 1) ctx->small_burst = mb << 20;
+    }
     ctx->small_workers = std::min(cfg.n_threads, std::max(4u, cfg.n_threads * 3 / 4));
     if (const char *e = std::getenv("FSTX_SMALL_WORKERS")) {
         const uint64_t n = std::strtoull(e, nullptr, 10);
@@ -1750,7 +1756,7 @@ int64_t fstx_submit_read(fstx_ctx *ctx, int64_t file, uint64_t file_off, uint64_
         std::lock_guard<std::mutex> lk(ctx->q_mutex);
         if (ctx->queue.empty() && ctx->staged.empty()) ctx->burst_bytes = 0;
         ctx->burst_bytes += length;
-        req->small = ctx->burst_bytes < kSmallRequest;
+        req->small = ctx->burst_bytes < ctx->small_burst;
     }
     if (file_off > req->file->size || length > req->file->size - file_off)
         req->error.store(-FSTX_E_SHORT_READ); // reported by wait_read, like a failed read

@@ -621,3 +621,34 @@ def test_a_context_that_failed_parks_nothing(sim, monkeypatch):
         assert sim.fstx_cached_ring_bytes() == 0 and sim.fstx_sim_pinned_live() == 0
     finally:
         sim.fstx_sim_fail_host_allocs(0)
+
+
+def test_only_the_first_bytes_of_a_burst_are_cut_small(sim, blob, monkeypatch):
+    """Requests are cut into small blocks while little has been submitted since the reader was
+    last found idle; what follows in the same burst gets whole blocks.  Counted in blocks: a
+    4 MiB limit, 1 MiB small blocks, 4 MiB blocks, one worker whose first copy takes long enough
+    for the other submits to find its blocks still queued."""
+    path, data = blob
+    monkeypatch.setenv("FSTX_SMALL_BURST_MB", "4")
+    monkeypatch.setenv("FSTX_SMALL_BLOCK_KB", "1024")
+    sim.fstx_sim_set_copy_delay_us(50_000)
+    try:
+        ctx = make_ctx(sim, block=4 << 20, threads=1, slots=1)
+        f = sim.fstx_file_open(ctx, path.encode(), _native.READ_BUFFERED)
+        dev = np.zeros(data.size, dtype=np.uint8)
+        three = (2 << 20) + (512 << 10)  # (the file has 8.6 MiB)
+        reqs = [sim.fstx_submit_read(ctx, f, k * three, three, dev.ctypes.data, dev.size, k * three) for k in range(3)]
+        for r in reqs:
+            assert sim.fstx_wait_read(ctx, r) == three
+        assert np.array_equal(dev[: 3 * three], data[: 3 * three])
+        # 2.5 MiB under the limit: blocks of 1, 1 and 0.5 MiB; then 5 and 7.5 MiB submitted: whole blocks,
+        # cut on 4 MiB boundaries counted from the start of each request (one block each)
+        assert metrics(sim, ctx).blocks_buffered == 3 + 1 + 1
+        # idle again: the count starts over
+        r = sim.fstx_submit_read(ctx, f, 0, three, dev.ctypes.data, dev.size, 0)
+        assert sim.fstx_wait_read(ctx, r) == three
+        assert metrics(sim, ctx).blocks_buffered == 5 + 3
+        assert sim.fstx_file_close(ctx, f) == 0
+        assert sim.fstx_ctx_destroy(ctx) == 0
+    finally:
+        sim.fstx_sim_set_copy_delay_us(30)
