@@ -1067,15 +1067,25 @@ def bench_whole_load(files: List[str], data_bytes: int, verify, threads: int, bl
     verified against the generator's checksums.  ``iterate`` adds ``ParallelLoader.iterate_weights``."""
     import torch
 
-    runs = [run_load(files, "auto", threads, block_kb, verify if i == 0 else None) for i in range(reps)]
-    # best of three, and on the device memory the loads have just returned to the allocator: a leg
-    # is a ceiling, and a pass over device memory that was never handed out before runs 10 % slower
-    leg = max((engine_leg(files, "copy_only", threads, block_kb) for _ in range(3)), key=lambda r: r["GBps"])
-    torch.cuda.empty_cache()
+    # Loads and legs take turns, best of each, on the device memory the pass before has just returned
+    # to the allocator: a leg is a ceiling, and a pass over device memory that was never handed out
+    # before runs 10 % slower.  A leg that a load has beaten is no ceiling: up to three more are taken.
+    runs = [run_load(files, "auto", threads, block_kb, verify)]
+    legs = []
+    for _ in range(max(reps - 1, 1)):
+        legs.append(engine_leg(files, "copy_only", threads, block_kb))
+        runs.append(run_load(files, "auto", threads, block_kb, None))
     best = min(runs, key=lambda r: r["elapsed_s"])
+    for _ in range(3):
+        if max(r["GBps"] for r in legs) >= data_bytes / 1e9 / best["elapsed_s"]:
+            break
+        legs.append(engine_leg(files, "copy_only", threads, block_kb))
+    leg = max(legs, key=lambda r: r["GBps"])
+    torch.cuda.empty_cache()
     out = {"files": len(files), "data_bytes": data_bytes, "seconds_to_load": best["elapsed_s"],
            "seconds_all": [r["elapsed_s"] for r in runs], "GBps": data_bytes / 1e9 / best["elapsed_s"],
-           "copy_only_leg_GBps": leg["GBps"], "frac_of_copy_only_leg": data_bytes / 1e9 / best["elapsed_s"] / leg["GBps"],
+           "copy_only_leg_GBps": leg["GBps"], "copy_only_legs_all_GBps": [r["GBps"] for r in legs],
+           "frac_of_copy_only_leg": data_bytes / 1e9 / best["elapsed_s"] / leg["GBps"],
            "verified_tensors": runs[0].get("verified_tensors", 0)}
     if iterate:
         out["iterate_weights"] = bench_iterate_weights(files, threads, verify)
@@ -1486,6 +1496,11 @@ def main() -> None:
             line["configs"]["C5"]["cpu_reference_sample"] = c5["cpu_reference"]["sample"]
     else:
         line["configs"]["C5"] = c5
+    for key, whole in (("C4", c4), ("C5", c5)):
+        if whole.get("frac_of_copy_only_leg", 0) > 1.0:
+            # the leg fell into a slow stretch of the link (they come and go within seconds): it bounds nothing here
+            line["configs"][key]["copy_only_leg_valid"] = False
+            line["configs"][key]["copy_only_legs_GBps"] = [r3(x) for x in whole["copy_only_legs_all_GBps"]]
     line["downcast_on_load_GBps"] = {k: r3(v["GBps"]) for k, v in downcast.items() if isinstance(v, dict)}
     line["placement"] = placement
     line["inputs"] = {k: {"generator_device": v["generator_device"], "seed_base": v["seed_base"],
