@@ -1497,8 +1497,9 @@ def main() -> None:
     else:
         line["configs"]["C5"] = c5
     for key, whole in (("C4", c4), ("C5", c5)):
-        if whole.get("frac_of_copy_only_leg", 0) > 1.0:
-            # the leg fell into a slow stretch of the link (they come and go within seconds): it bounds nothing here
+        if whole.get("frac_of_copy_only_leg", 0) > 1.01:
+            # (up to 1 % is the scatter of two passes at the link's rate.)  Beyond that the legs fell into
+            # a slow stretch of the link (they come and go within seconds) and bound nothing here
             line["configs"][key]["copy_only_leg_valid"] = False
             line["configs"][key]["copy_only_legs_GBps"] = [r3(x) for x in whole["copy_only_legs_all_GBps"]]
     line["downcast_on_load_GBps"] = {k: r3(v["GBps"]) for k, v in downcast.items() if isinstance(v, dict)}
