@@ -320,6 +320,7 @@ class cpp_metrics:
 
     def __init__(self) -> None:
         self.bounce_buffer_bytes = bounce_buffer_bytes()
+        self.cached_ring_bytes = cached_ring_bytes()  # the ring a closed reader left for the next one
 
 
 def get_cpp_metrics() -> cpp_metrics:
