@@ -202,6 +202,70 @@ def test_a_closed_readers_ring_serves_the_next_reader(golden):
     assert _native.cached_ring_bytes() == 0 and fastsafetensors_amd.release_cached_memory() == 0
 
 
+def test_random_settings_load_the_same_bytes(tmp_path, monkeypatch):
+    """Sixty loads of one small multi-file checkpoint with settings drawn at random -- threads,
+    block size, read mode, layout, private or shared reader, page cache dropped or not, the ring
+    of the last reader kept or not, two loaders at once now and then: every tensor has the
+    checksum of the first load, whose bytes are compared with the oracle's."""
+    import random
+    import threading
+
+    import fastsafetensors_amd
+
+    cfg = ck.configs(0.02)["C3"]
+    files = [r["path"] for r in ck.write_config(cfg, str(tmp_path / "c3"))]
+    loader = SafeTensorsFileLoader(SingleGroup(), DEV, max_threads=4)
+    loader.add_filenames({0: files})
+    bufs = loader.copy_files_to_device()
+    want = {}
+    for path in files:
+        h = orc.parse_file(path)
+        for name in h.tensors:
+            t = bufs.get_tensor(name)
+            assert np.array_equal(dev_bytes(t), orc.tensor_bytes(path, h, name)), name
+            want[name] = ck.tensor_checksum(t)
+    bufs.close()
+    loader.close()
+    rng = random.Random(11)
+    bad = []
+
+    def one(kw, subset):
+        ld = SafeTensorsFileLoader(SingleGroup(), DEV, **kw)
+        ld.add_filenames({0: subset})
+        b = ld.copy_files_to_device()
+        bad.extend((kw, k) for k in ld.get_keys() if ck.tensor_checksum(b.get_tensor(k)) != want[k])
+        b.close()
+        ld.close()
+
+    def draw():
+        return dict(max_threads=rng.choice([1, 2, 3, 8, 16]), block_size_kb=rng.choice([64, 256, 1024, 4096]),
+                    read_mode=rng.choice(["auto", "buffered", "direct"]), layout=rng.choice(["direct", "window"]),
+                    shared_reader=rng.choice([True, False])), (files if rng.random() < 0.7 else files[:1])
+
+    for i in range(60):
+        monkeypatch.setenv("FSTX_RING_CACHE", rng.choice(["0", "1", "1"]))
+        if rng.random() < 0.3:
+            for p in files:
+                fd = os.open(p, os.O_RDONLY)
+                os.fsync(fd)
+                os.posix_fadvise(fd, 0, 0, os.POSIX_FADV_DONTNEED)
+                os.close(fd)
+        if i % 5 == 4:
+            pair = [threading.Thread(target=one, args=draw()) for _ in range(2)]
+            for t in pair:
+                t.start()
+            for t in pair:
+                t.join()
+        else:
+            one(*draw())
+        assert not bad, bad[:3]
+        assert_clean()
+        if i % 9 == 8:
+            fastsafetensors_amd.release_cached_memory()
+    fastsafetensors_amd.release_cached_memory()
+    assert _native.cached_ring_bytes() == 0
+
+
 def test_adaptive_depth_and_small_direct_reads(tmp_path):
     """O_DIRECT with many small reads in flight and the depth steered while reading -- the
     setting for storage that wants a deep queue -- byte-exact against the oracle."""
