@@ -487,6 +487,7 @@ struct fstx_ctx {
     StorageFacts storage;
     int ring_node = -1;        // node of the ring's first page, where the kernel says (ready_mutex)
     bool ring_reused = false;  // the ring is the one an earlier context of this process left behind
+    bool ring_cache = true;    // take over a parked ring, and leave this one parked (the environment, read when the context is created)
     uint64_t direct_bytes = 0; // bytes one O_DIRECT pread may cover
     // ordinary page-backed blocks that O_DIRECT reads land in; handed out together
     // with the read token (under q_mutex), returned after the last byte left for the ring
@@ -1222,7 +1223,6 @@ bool ring_cache_on() {
 
 // the parked ring, if it fits; the caller owns it from here on
 bool take_parked(int device, int node, uint64_t bytes, ParkedRing &out) {
-    if (!ring_cache_on()) return false;
     std::lock_guard<std::mutex> lk(g_park_mutex);
     if (!g_parked.p || g_parked.device != device || g_parked.node != node || g_parked.bytes != bytes) return false;
     out = std::move(g_parked);
@@ -1233,7 +1233,7 @@ bool take_parked(int device, int node, uint64_t bytes, ParkedRing &out) {
 // leaves the ring of a context behind for the next one (replacing what is parked), or frees it
 void park_or_free_ring(fstx_ctx *ctx) {
     ParkedRing old;
-    if (ring_cache_on() && ctx->build_status == 0 && !ctx->failed) {
+    if (ctx->ring_cache && ctx->build_status == 0 && !ctx->failed) {
         ParkedRing mine;
         mine.p = ctx->ring;
         mine.bytes = ctx->ring_bytes;
@@ -1369,7 +1369,7 @@ int build_context(fstx_ctx *ctx) {
         if (own_thread) bound = bind_thread_to_node(cfg.numa_node); // never the caller's own affinity and policy
         ring_rc = fstx_dev::set_device(cfg.device_id);
         ParkedRing parked;
-        if (ring_rc == 0 && take_parked(cfg.device_id, cfg.numa_node, ctx->ring_bytes, parked)) {
+        if (ring_rc == 0 && ctx->ring_cache && take_parked(cfg.device_id, cfg.numa_node, ctx->ring_bytes, parked)) {
             // the ring an earlier context left behind: allocated, placed, and mapped where it was used
             p = parked.p;
             ring_node = parked.ring_node;
@@ -1550,6 +1550,7 @@ int fstx_ctx_create(const fstx_config *cfg_in, fstx_ctx **out) {
 
     // measured on 0.5 and 0.7 GB files in the page cache: twelve workers with one slot each beat
     // eight with two by 4 to 6 % (12 MiB of pinned memory to map before the link runs, not 16)
+    ctx->ring_cache = ring_cache_on();
     ctx->small_burst = kSmallRequest;
     if (const char *e = std::getenv("FSTX_SMALL_BURST_MB")) {
         const uint64_t mb = std::strtoull(e, nullptr, 10);

@@ -193,7 +193,8 @@ uint64_t fstx_bounce_buffer_bytes(void);
  * (the reference allocates its bounce buffer per reader, nogds.py:107-116 / ext.cpp:648-672, and
  * pays that every time).  At most one ring is parked; it is not counted by
  * fstx_bounce_buffer_bytes.  fstx_cached_ring_bytes tells its size, fstx_trim_cache frees it
- * (returns the bytes freed); with FSTX_RING_CACHE=0 in the environment nothing is ever parked.
+ * (returns the bytes freed); a context created with FSTX_RING_CACHE=0 in the environment neither
+ * takes over a parked ring nor leaves its own behind.
  * No counterpart in the reference. */
 uint64_t fstx_cached_ring_bytes(void);
 uint64_t fstx_trim_cache(void);
