@@ -140,7 +140,6 @@ class MI355XFileCopier(CopierInterface):
     ) -> Dict[str, TensorBase]:
         meta, fw = self.metadata, self.framework
         if dtype != DType.AUTO and any(f.dtype != dtype for f in meta.tensors.values()):
-            self._drain_or_raise()
             return self._converted(gbuf, dtype)
 
         # Everything that does not need the bytes happens while they are still on their way: where
@@ -214,6 +213,7 @@ class MI355XFileCopier(CopierInterface):
         for name, frame in meta.tensors.items():
             if frame.dtype != dtype and frame.nbytes:
                 if want_bits > dtype_bits(frame.dtype):
+                    self._drain()  # nothing may still be writing to the arena when the caller frees it
                     raise Exception(
                         f"Online type conversion to larger sizes is not supported ({frame.dtype} -> {dtype})"
                     )
@@ -234,12 +234,8 @@ class MI355XFileCopier(CopierInterface):
                 scratch_bytes += _align_up(frame.nbytes, LINE_ALIGN)
         scratch = fw.alloc_tensor_memory(scratch_bytes, self.device) if staged else None
         try:
-            if staged:
-                _native.realign_copy_batch(
-                    [(scratch.get_base_address() + at, src_at + meta.tensors[n].data_offsets[0], meta.tensors[n].nbytes)
-                     for n, at in staged.items()],
-                    self._stream(),
-                )
+            # Everything up to here and the views below need no byte of the file: it all happens
+            # while the bytes are still on their way; the kernels follow the wait.
             convert, copy, by_framework = [], [], []
             for name, at in placed.items():
                 frame = meta.tensors[name]
@@ -254,6 +250,25 @@ class MI355XFileCopier(CopierInterface):
                                     _native.ELEM_TYPES[frame.dtype.value], _native.ELEM_TYPES[dtype.value]))
                 else:
                     by_framework.append((name, at))
+            tensors: Dict[str, TensorBase] = {}
+            for name, frame in meta.tensors.items():
+                if name in placed:
+                    if frame.dtype != dtype:
+                        count = frame.nbytes * 8 // dtype_bits(frame.dtype)
+                        # a frame of its own for the view: the header model keeps describing the file
+                        frame = TensorFrame(dtype, frame.shape, [placed[name], placed[name] + count * want_bits // 8],
+                                            frame.strides, frame.offsets, frame.sliced)
+                    tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
+                else:
+                    tensors[name] = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)
+
+            self._drain_or_raise()
+            if staged:
+                _native.realign_copy_batch(
+                    [(scratch.get_base_address() + at, src_at + meta.tensors[n].data_offsets[0], meta.tensors[n].nbytes)
+                     for n, at in staged.items()],
+                    self._stream(),
+                )
             _native.convert_batch(convert, self._stream())
             _native.realign_copy_batch(copy, self._stream())
             # Pairs the conversion kernel does not cover (integer and bool tensors, fp8 sources)
@@ -261,28 +276,14 @@ class MI355XFileCopier(CopierInterface):
             # every tensor (common.py:355-375).
             for name, at in by_framework:
                 frame = meta.tensors[name]
-                count = frame.nbytes * 8 // dtype_bits(frame.dtype)
                 if name in staged:
                     src_view = fw.view_tensor(scratch, staged[name], frame, self.device)
                 else:
                     src_view = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)
-                out_frame = TensorFrame(dtype, frame.shape, [at, at + count * want_bits // 8],
-                                        frame.strides, frame.offsets, frame.sliced)
-                fw.copy_tensor(fw.view_tensor(side, at, out_frame, self.device), src_view)
+                fw.copy_tensor(tensors[name], src_view)
         finally:
             if scratch is not None:
                 fw.free_tensor_memory(scratch, self.device)  # reuse is ordered after the kernels above on this stream
-        tensors: Dict[str, TensorBase] = {}
-        for name, frame in meta.tensors.items():
-            if name in placed:
-                if frame.dtype != dtype:
-                    count = frame.nbytes * 8 // dtype_bits(frame.dtype)
-                    # a frame of its own for the view: the header model keeps describing the file
-                    frame = TensorFrame(dtype, frame.shape, [placed[name], placed[name] + count * want_bits // 8],
-                                        frame.strides, frame.offsets, frame.sliced)
-                tensors[name] = fw.view_tensor(side, placed[name], frame, self.device)
-            else:
-                tensors[name] = fw.view_tensor(gbuf, self.data_at + frame.data_offsets[0], frame, self.device)
         if len(placed) == len(meta.tensors):
             fw.shrink_tensor_memory(gbuf)  # nothing lives in the original arena any more
         return tensors
